@@ -1,0 +1,427 @@
+// diopiContextAttentionInference for gfx950: causal softmax(q k^T / sqrt(D)) v over packed
+// variable-length sequences.
+//
+// Semantics: impl/torch/functions/functions_lightllm.cpp:109-147 of the reference (Python statement
+// customized_test.py:8-33, 735-749).  Sequence i owns rows [b_start_loc[i], b_start_loc[i] + b_seq_len[i])
+// of q, k, v and out ([rows, H, D]); inside a sequence, query row r attends to key rows 0..r.  The
+// reference materialises an L x L score matrix per head, rounds it to the element type, applies an
+// fp32 softmax and rounds the probabilities to the element type before the product with V.  This
+// kernel keeps the fp32 scores in registers (online softmax, O(L) memory) and rounds only the
+// probabilities, which stays inside the reference's 16-bit tolerance.  Rows outside every sequence
+// are not written; max_input_len is not needed (the reference never reads it either).
+//
+// MFMA kernel (fp16 / bf16, D == 128).  One 256-thread work-group owns 128 query rows of one
+// (sequence, head); each of its four waves owns 32 of them.  Key/value tiles of 64 rows are staged
+// row-major in LDS and shared by the four waves.  Everything is computed transposed so that no
+// cross-lane data movement is needed between the two matrix products:
+//   S^T[key, q]  = K[key, :] . Q[q, :]      v_mfma_f32_32x32x16, A = K rows from LDS, B = Q rows (registers)
+//   O^T[d, q]   += V^T[d, key] . P^T[key, q]                    A = V columns from LDS, B = P^T
+// In the 32x32 accumulator layout a lane holds one query column, so the row maximum, the row sum
+// and the rescaling of O^T are per-lane scalars (one exchange with lane ^ 32 per tile), and the
+// exponentiated scores are already in the B-operand layout of the second product.
+// Work-groups are numbered so that the query tiles of one head land on the same XCD (they share
+// that head's K/V through its L2), and the heaviest (last) query tiles of a sequence start first.
+#include <cmath>
+
+#include "common.hpp"
+#include "device.hpp"
+
+namespace rocm {
+namespace {
+
+constexpr int kCtxThreads = 256;
+constexpr int kBM = 128;   // query rows per work-group
+constexpr int kBN = 64;    // key rows per tile
+constexpr int kHD = 128;   // head size of the MFMA kernel
+constexpr int kLD = kHD + 8;  // LDS row pitch in elements (272 bytes: 16-byte aligned, conflict-free 128-bit reads)
+constexpr int kNumXcd = 8;
+
+struct CtxArgs {
+    const void* bStartLoc;
+    const void* bSeqLen;
+    bool start64, len64;
+    int batch;
+    int H;
+    int64_t rows;      // rows of q / k / v / out
+    int tilesBound;    // upper bound on the number of 128-row query tiles over all sequences
+    int totalItems;    // H * tilesBound
+};
+
+template <typename T>
+struct Mfma32;
+template <>
+struct Mfma32<half_t> {
+    using Frag = f16x8;
+    static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <>
+struct Mfma32<bf16_t> {
+    using Frag = bf16x8;
+    static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+
+template <typename Frag>
+union FragBits {
+    u32x4 raw;
+    Frag f;
+    __device__ FragBits() {}
+};
+
+// Sequence geometry with every value forced inside the tensors.
+struct SeqInfo {
+    int64_t start;
+    int64_t len;
+};
+
+__device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
+    SeqInfo s;
+    s.start = loadIndex(a.bStartLoc, i, a.start64);
+    s.len = loadIndex(a.bSeqLen, i, a.len64);
+    if (s.start < 0 || s.start >= a.rows) s.len = 0;
+    if (s.len > a.rows - s.start) s.len = a.rows - s.start;
+    if (s.len < 0) s.len = 0;
+    return s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                                               CtxArgs a, float scaleLog2) {
+    using Ops = Mfma32<T>;
+    using Frag = typename Ops::Frag;
+    __shared__ __attribute__((aligned(16))) T smem[2 * kBN * kLD];
+    T* sK = smem;
+    T* sV = smem + kBN * kLD;
+
+    // ---- which (head, sequence, query tile) is this work-group? ----
+    const int perXcd = (a.totalItems + kNumXcd - 1) / kNumXcd;
+    const int item = (blockIdx.x % kNumXcd) * perXcd + blockIdx.x / kNumXcd;
+    if (item >= a.totalItems) return;
+    const int head = item / a.tilesBound;
+    const int tileFlat = item % a.tilesBound;
+    int seq = 0, before = 0, numTiles = 0;
+    SeqInfo si{0, 0};
+    for (; seq < a.batch; ++seq) {
+        si = loadSeq(a, seq);
+        numTiles = static_cast<int>((si.len + kBM - 1) / kBM);
+        if (tileFlat < before + numTiles) break;
+        before += numTiles;
+    }
+    if (seq >= a.batch) return;
+    const int qt = numTiles - 1 - (tileFlat - before);  // last (longest) tiles first
+    const int64_t L = si.len;
+    const int64_t m0 = static_cast<int64_t>(qt) * kBM;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int n = lane % 32;   // query column of this lane in every accumulator
+    const int hh = lane / 32;  // which half of the k slots / which 4-row sub-block of the accumulator
+    const int64_t rowPitch = static_cast<int64_t>(a.H) * kHD;
+    const T* qBase = q + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+    const T* kBase = k + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+    const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+
+    // ---- Q fragments (B operand of S^T): row = m0 + 32*wave + n, k slot (hh, e) <-> dim 16*s + 8*hh + e ----
+    const int64_t qRow = m0 + wave * 32 + n;
+    const int64_t qRowLd = qRow < L ? qRow : L - 1;
+    Frag qf[kHD / 16];
+#pragma unroll
+    for (int s = 0; s < kHD / 16; ++s) {
+        FragBits<Frag> u;
+        u.raw = *reinterpret_cast<const u32x4*>(qBase + qRowLd * rowPitch + s * 16 + hh * 8);
+        qf[s] = u.f;
+    }
+
+    f32x16 o[kHD / 32];
+#pragma unroll
+    for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[mb][r] = 0.f;
+    }
+    float mRun = -1e30f;
+    float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
+
+    const int64_t kEnd = (m0 + kBM < L) ? m0 + kBM : L;  // keys 0 .. kEnd-1 are visible to this tile
+    const int numKeyTiles = static_cast<int>((kEnd + kBN - 1) / kBN);
+    const int64_t waveRowLo = m0 + wave * 32;
+    const int64_t waveRowHi = waveRowLo + 31;
+
+    // tile staging: thread -> 16-byte packet ldC of rows ldR, ldR+16, ldR+32, ldR+48
+    const int ldC = tid % 16;
+    const int ldR = tid / 16;
+    u32x4 kReg[4], vReg[4];
+    auto loadTile = [&](int jt) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            int64_t row = static_cast<int64_t>(jt) * kBN + ldR + it * 16;
+            if (row > L - 1) row = L - 1;  // keeps the load in bounds; such keys are masked below
+            kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
+            vReg[it] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
+        }
+    };
+    loadTile(0);
+
+    for (int jt = 0; jt < numKeyTiles; ++jt) {
+        __syncthreads();  // every wave is done with the previous tile
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            *reinterpret_cast<u32x4*>(sK + (ldR + it * 16) * kLD + ldC * 8) = kReg[it];
+            *reinterpret_cast<u32x4*>(sV + (ldR + it * 16) * kLD + ldC * 8) = vReg[it];
+        }
+        __syncthreads();
+        if (jt + 1 < numKeyTiles) loadTile(jt + 1);  // in flight while this tile is computed
+
+        const int64_t key0 = static_cast<int64_t>(jt) * kBN;
+        if (key0 > waveRowHi) continue;  // entirely above the diagonal for this wave (barriers are at the loop top)
+
+        // ---- S^T = K . Q^T for the two 32-key blocks ----
+        f32x16 s[2];
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
+#pragma unroll
+            for (int st = 0; st < kHD / 16; ++st) {
+                FragBits<Frag> u;
+                u.raw = *reinterpret_cast<const u32x4*>(sK + (sb * 32 + n) * kLD + st * 16 + hh * 8);
+                s[sb] = Ops::mma(u.f, qf[st], s[sb]);
+            }
+        }
+        // accumulator register r of block sb holds key  key0 + 32*sb + 8*(r/4) + 4*hh + r%4  for query row qRow
+        if (key0 + kBN - 1 > waveRowLo) {
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t key = key0 + sb * 32 + (r / 4) * 8 + hh * 4 + (r % 4);
+                    if (key > qRow) s[sb][r] = -1e30f;
+                }
+            }
+        }
+        float tmax = -1e30f;
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[sb][r]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float mNew = fmaxf(mRun, tmax);
+        const float alpha = __builtin_amdgcn_exp2f((mRun - mNew) * scaleLog2);
+        const float mc = mNew * scaleLog2;
+        mRun = mNew;
+        float psum = 0.f;
+        Frag pf[2][2];
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
+                    psum += p;
+                    pf[sb][u][j] = static_cast<T>(p);
+                }
+            }
+        }
+        lRun = lRun * alpha + psum;
+#pragma unroll
+        for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[mb][r] *= alpha;
+        }
+        // ---- O^T += V^T . P^T : k slot (hh, j) of step (sb, u) is key 32*sb + 16*u + 8*(j/4) + 4*hh + j%4 ----
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int mb = 0; mb < kHD / 32; ++mb) {
+                    Frag vf;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int key = sb * 32 + u * 16 + (j / 4) * 8 + hh * 4 + (j % 4);
+                        vf[j] = sV[key * kLD + mb * 32 + n];
+                    }
+                    o[mb] = Ops::mma(vf, pf[sb][u], o[mb]);
+                }
+            }
+        }
+    }
+
+    // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
+    const float lTot = lRun + __shfl_xor(lRun, 32, kWave);
+    const float inv = 1.0f / lTot;
+    __syncthreads();  // the K/V tiles are dead; reuse the storage as a [128][kLD] output tile
+    T* sO = smem;
+#pragma unroll
+    for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            // registers 4*r4 .. 4*r4+3 are dims 32*mb + 8*r4 + 4*hh + 0..3 of query row (32*wave + n)
+            T pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = static_cast<T>(o[mb][r4 * 4 + e] * inv);
+            *reinterpret_cast<u32x2*>(sO + (wave * 32 + n) * kLD + mb * 32 + r4 * 8 + hh * 4) = *reinterpret_cast<const u32x2*>(pk);
+        }
+    }
+    // each wave only reads back the 32 rows it wrote: no work-group barrier needed, LDS ops of a wave are ordered
+    T* oBase = out + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int id = it * kWave + lane;
+        const int row = id / 16;
+        const int c = id % 16;
+        const int64_t grow = m0 + wave * 32 + row;
+        if (grow < L) {
+            const u32x4 val = *reinterpret_cast<const u32x4*>(sO + (wave * 32 + row) * kLD + c * 8);
+            *reinterpret_cast<u32x4*>(oBase + grow * rowPitch + c * 8) = val;
+        }
+    }
+}
+
+// Any dtype / head size up to 512: one wave per (query row, head); lanes split the head dimension.
+template <typename T, typename AccT>
+__global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, CtxArgs a,
+                                                        int D, AccT scale) {
+    constexpr int kPerLane = 8;
+    const int head = blockIdx.y;
+    const int64_t grow = blockIdx.x;  // row of the packed tensors
+    // find the sequence that owns this row
+    int seq = 0;
+    SeqInfo si{0, 0};
+    for (; seq < a.batch; ++seq) {
+        si = loadSeq(a, seq);
+        if (grow >= si.start && grow < si.start + si.len) break;
+    }
+    if (seq >= a.batch) return;
+    const int64_t r = grow - si.start;
+    const int lane = threadIdx.x;
+    const int64_t rowPitch = static_cast<int64_t>(a.H) * D;
+    const T* qRow = q + grow * rowPitch + static_cast<int64_t>(head) * D;
+    AccT qv[kPerLane], acc[kPerLane];
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) {
+        const int d = lane + e * kWave;
+        qv[e] = d < D ? static_cast<AccT>(qRow[d]) : static_cast<AccT>(0);
+        acc[e] = 0;
+    }
+    AccT m = static_cast<AccT>(-INFINITY), l = 0;
+    for (int64_t j = 0; j <= r; ++j) {
+        const T* kRow = k + (si.start + j) * rowPitch + static_cast<int64_t>(head) * D;
+        const T* vRow = v + (si.start + j) * rowPitch + static_cast<int64_t>(head) * D;
+        AccT part = 0;
+#pragma unroll
+        for (int e = 0; e < kPerLane; ++e) {
+            const int d = lane + e * kWave;
+            if (d < D) part += qv[e] * static_cast<AccT>(kRow[d]);
+        }
+        const AccT sc = waveSum(part) * scale;
+        const AccT mNew = sc > m ? sc : m;
+        const AccT alpha = static_cast<AccT>(exp(static_cast<double>(m - mNew)));
+        const AccT p = static_cast<AccT>(exp(static_cast<double>(sc - mNew)));
+        l = l * alpha + p;
+#pragma unroll
+        for (int e = 0; e < kPerLane; ++e) {
+            const int d = lane + e * kWave;
+            if (d < D) acc[e] = acc[e] * alpha + p * static_cast<AccT>(vRow[d]);
+        }
+        m = mNew;
+    }
+    T* oRow = out + grow * rowPitch + static_cast<int64_t>(head) * D;
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) {
+        const int d = lane + e * kWave;
+        if (d < D) oRow[d] = static_cast<T>(acc[e] / l);
+    }
+}
+
+template <typename T>
+diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
+    a.tilesBound = static_cast<int>(ceilDiv(a.rows, kBM)) + a.batch;
+    const int64_t total = static_cast<int64_t>(a.tilesBound) * a.H;
+    ROCM_CHECK(total < INT32_MAX / 2, "context attention: too many tiles for one launch");
+    a.totalItems = static_cast<int>(total);
+    const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
+    // exp(x) = exp2(x * log2(e)); the 1/sqrt(D) scaling of the scores is folded into the same factor
+    const float scaleLog2 = static_cast<float>(1.4426950408889634 / std::sqrt(static_cast<double>(kHD)));
+    hipLaunchKernelGGL(ctxAttnMfma<T>, dim3(grid), dim3(kCtxThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
+                       static_cast<const T*>(v), a, scaleLog2);
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
+template <typename T, typename AccT>
+diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const void* v, const CtxArgs& a, int D) {
+    ROCM_CHECK(D <= 8 * kWave, "context attention: head size %d is not supported (at most %d)", D, 8 * kWave);
+    ROCM_CHECK(a.H <= 65535, "context attention: %d heads exceed the launch limit", a.H);
+    ROCM_CHECK(a.rows <= INT32_MAX, "context attention: too many rows for one launch");
+    const AccT scale = static_cast<AccT>(1.0 / std::sqrt(static_cast<double>(D)));
+    hipLaunchKernelGGL((ctxAttnGeneric<T, AccT>), dim3(static_cast<unsigned>(a.rows), static_cast<unsigned>(a.H)), dim3(kWave), 0, stream,
+                       static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v), a, D, scale);
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
+}  // namespace
+}  // namespace rocm
+
+extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
+                                                       diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
+                                                       diopiConstTensorHandle_t b_seq_len, int max_input_len) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)max_input_len;  // never read by the reference (functions_lightllm.cpp:127-147); lengths come from b_seq_len
+    TensorView vOut, vQ, vK, vV, vStart, vLen;
+    ROCM_CALL(unwrap(context_attention_out, "context_attention_out", &vOut));
+    ROCM_CALL(unwrap(q, "q", &vQ));
+    ROCM_CALL(unwrap(k, "k", &vK));
+    ROCM_CALL(unwrap(v, "v", &vV));
+    ROCM_CALL(unwrap(b_start_loc, "b_start_loc", &vStart));
+    ROCM_CALL(unwrap(b_seq_len, "b_seq_len", &vLen));
+    ROCM_CALL(requireDeviceContiguous(vOut, "context_attention_out"));
+    ROCM_CALL(requireDeviceContiguous(vQ, "q"));
+    ROCM_CALL(requireDeviceContiguous(vK, "k"));
+    ROCM_CALL(requireDeviceContiguous(vV, "v"));
+    ROCM_CALL(requireDeviceContiguous(vStart, "b_start_loc"));
+    ROCM_CALL(requireDeviceContiguous(vLen, "b_seq_len"));
+    ROCM_CHECK(vQ.ndim == 3, "q must be [rows, heads, head_dim], got rank %d", vQ.ndim);
+    ROCM_CHECK(vK.sameShape(vQ) && vV.sameShape(vQ) && vOut.sameShape(vQ), "q, k, v and out must have identical shapes (the reference has no grouped heads here)");
+    ROCM_CHECK(isFloatDtype(vQ.dtype) && vK.dtype == vQ.dtype && vV.dtype == vQ.dtype && vOut.dtype == vQ.dtype,
+               "q, k, v and out must share one floating dtype (q is %s)", dtypeName(vQ.dtype));
+    ROCM_CHECK(vStart.ndim == 1 && vLen.ndim == 1 && vStart.shape[0] == vLen.shape[0], "b_start_loc and b_seq_len must be 1-D of equal length");
+    ROCM_CHECK(isIndexDtype(vStart.dtype) && isIndexDtype(vLen.dtype), "b_start_loc and b_seq_len must be int32 or int64");
+    ROCM_CHECK(vStart.shape[0] <= 65535 && vQ.shape[1] <= INT32_MAX / 1024 && vQ.shape[2] <= 65535, "batch / head count / head size out of range");
+    if (vQ.numel == 0 || vStart.shape[0] == 0) return diopiSuccess;
+
+    CtxArgs a;
+    a.bStartLoc = vStart.data;
+    a.bSeqLen = vLen.data;
+    a.start64 = vStart.dtype == diopi_dtype_int64;
+    a.len64 = vLen.dtype == diopi_dtype_int64;
+    a.batch = static_cast<int>(vStart.shape[0]);
+    a.H = static_cast<int>(vQ.shape[1]);
+    a.rows = vQ.shape[0];
+    a.tilesBound = 0;
+    a.totalItems = 0;
+    const int D = static_cast<int>(vQ.shape[2]);
+
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    const bool aligned =
+        ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
+    const bool fast = D == kHD && aligned && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    switch (vQ.dtype) {
+        case diopi_dtype_float16:
+            return fast ? launchMfma<half_t>(stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                        : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
+        case diopi_dtype_bfloat16:
+            return fast ? launchMfma<bf16_t>(stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                        : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
+        case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
+        case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
+        default: break;
+    }
+    setLastError("diopiContextAttentionInference: dtype %s is not supported", dtypeName(vQ.dtype));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}

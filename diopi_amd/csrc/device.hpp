@@ -1,0 +1,121 @@
+// Device-side building blocks for the gfx950 kernels: element types and their
+// fp32 conversions, 128-bit global accesses, wavefront (64-lane) reductions.
+#ifndef DIOPI_ROCM_CSRC_DEVICE_HPP_
+#define DIOPI_ROCM_CSRC_DEVICE_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace rocm {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+using half_t = _Float16;
+using bf16_t = __bf16;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// The arithmetic type a given element type accumulates in (fp32, or fp64 for fp64 data),
+// matching at::acc_type as used by the reference (layer_norm_cuda_kernel.cu:971).
+template <typename T>
+struct AccType {
+    using type = float;
+};
+template <>
+struct AccType<double> {
+    using type = double;
+};
+
+template <typename T>
+__device__ __forceinline__ float toFloat(T v) {
+    return static_cast<float>(v);
+}
+
+// Round-to-nearest-even conversion from fp32 to the element type.
+template <typename T>
+__device__ __forceinline__ T fromFloat(float v) {
+    return static_cast<T>(v);
+}
+
+// fp64 sums are narrowed through the accumulation type of the destination.
+template <typename T>
+__device__ __forceinline__ T fromDouble(double v) {
+    if constexpr (sizeof(T) == 8) {
+        return v;
+    } else {
+        return static_cast<T>(static_cast<float>(v));
+    }
+}
+
+// A 16-byte packet of elements, the unit of every vectorised global access.
+template <typename T>
+struct Pack16 {
+    static constexpr int N = 16 / sizeof(T);
+    union {
+        u32x4 raw;
+        T e[N];
+    };
+    __device__ __forceinline__ Pack16() {}
+};
+
+template <typename T>
+__device__ __forceinline__ Pack16<T> loadPack(const T* p) {
+    Pack16<T> v;
+    v.raw = *reinterpret_cast<const u32x4*>(p);
+    return v;
+}
+
+// Streaming variants: data that is touched once should not displace reusable lines.
+template <typename T>
+__device__ __forceinline__ Pack16<T> loadPackStream(const T* p) {
+    Pack16<T> v;
+    v.raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return v;
+}
+
+template <typename T>
+__device__ __forceinline__ void storePack(T* p, const Pack16<T>& v) {
+    *reinterpret_cast<u32x4*>(p) = v.raw;
+}
+
+template <typename T>
+__device__ __forceinline__ void storePackStream(T* p, const Pack16<T>& v) {
+    __builtin_nontemporal_store(v.raw, reinterpret_cast<u32x4*>(p));
+}
+
+// Butterfly reductions over the 64 lanes of a wavefront; every lane ends with the result.
+template <typename T>
+__device__ __forceinline__ T waveSum(T v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T waveMax(T v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        T o = __shfl_xor(v, off, kWave);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// Reads an index tensor element as int64 whatever its storage width.
+__device__ __forceinline__ int64_t loadIndex(const void* base, int64_t i, bool is64) {
+    return is64 ? reinterpret_cast<const int64_t*>(base)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(base)[i]);
+}
+
+}  // namespace rocm
+
+#endif  // DIOPI_ROCM_CSRC_DEVICE_HPP_

@@ -1,0 +1,637 @@
+// diopiRMSNorm / diopiRMSNormBackward for gfx950.
+//
+// Arithmetic follows the reference kernels in
+// impl/torch/functions/functions_ext/layer_norm_cuda_kernel.cu (cuApplyRMSNorm 321-378,
+// cuComputePartGradGammaBeta 451-518, cuComputeGradGammaBeta 520-570, cuComputeGradInput 572-717)
+// and the host wrappers in rmsnorm.cu:17-28, 85-108 and functions_ext.cpp:66-107:
+//
+//   n2 = prod(normalized_shape), n1 = numel / n2
+//   inv_rms[r] = rsqrt(sum_l x[r,l]^2 / n2 + eps)            accumulated in fp32 (fp64 for fp64 input)
+//   out[r,l]   = weight[l] * OutT(inv_rms[r] * x[r,l])       (+ bias[l], rounded again)
+//   g = dout * weight;  s[r] = sum_l g * x * inv_rms
+//   grad_input[r,l]  = (inv_rms / n2) * (n2 * g - x * inv_rms * s[r])
+//   grad_weight[l]   = sum_r dout[r,l] * x[r,l] * inv_rms[r]
+//   grad_bias[l]     = sum_r dout[r,l]
+//
+// Where this design departs from the reference's launch shapes (one 128-thread block per row with
+// scalar loads; grad_weight from a second full pass over x and dout):
+//  * forward: one 64-lane wavefront owns a row, holds it in registers as 16-byte packets, reduces
+//    with cross-lane shuffles only (no LDS, no barrier) and streams it back out: exactly one read
+//    and one write of the matrix.  The weight packets stay in registers across the rows a wave
+//    visits.
+//  * backward: one pass.  A 256-thread group walks rows; each thread keeps the columns it owns in
+//    registers for x and dout, the row sum s[r] is a single barrier away, and the column sums for
+//    grad_weight / grad_bias accumulate in registers across rows.  Per-group partial sums go to a
+//    context-owned scratch buffer and a small second kernel folds them.  x and dout are read once.
+//  * column sums are accumulated in fp64 when the data is fp32/fp64, which makes grad_weight
+//    independent of the summation order to well below fp32 rounding.
+#include <type_traits>
+
+#include "common.hpp"
+#include "device.hpp"
+
+namespace rocm {
+namespace {
+
+// ---------------------------------------------------------------------------
+// Forward, register-resident row: requires n2 * sizeof(TIn) to be a multiple of 16 bytes and at
+// most NV * 64 packets per row.
+// ---------------------------------------------------------------------------
+constexpr int kFwdThreads = 256;
+constexpr int kFwdWaves = kFwdThreads / kWave;
+
+template <typename TIn, typename TOut, int NV, bool HAS_BIAS>
+__global__ __launch_bounds__(kFwdThreads) void rmsNormFwdRowReg(TOut* __restrict__ out, float* __restrict__ invRms, const TIn* __restrict__ x,
+                                                                 const TOut* __restrict__ weight, const TOut* __restrict__ bias, int64_t n1, int n2,
+                                                                 float eps, int rowsPerWave) {
+    constexpr int EPV = Pack16<TIn>::N;  // elements per input packet
+    const int lane = threadIdx.x % kWave;
+    const int64_t waveId = static_cast<int64_t>(blockIdx.x) * kFwdWaves + threadIdx.x / kWave;
+    const int nvec = n2 / EPV;
+    int64_t row = waveId * rowsPerWave;
+    int64_t rowEnd = row + rowsPerWave;
+    if (rowEnd > n1) rowEnd = n1;
+    if (row >= rowEnd) return;
+
+    // weight (and bias) for the columns this lane owns, as fp32
+    float w[NV][EPV];
+    float b[NV][EPV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int v = j * kWave + lane;
+        if (v < nvec) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                w[j][e] = toFloat(weight[v * EPV + e]);
+                if (HAS_BIAS) b[j][e] = toFloat(bias[v * EPV + e]);
+            }
+        }
+    }
+
+    const float rn2 = 1.0f / static_cast<float>(n2);
+    for (; row < rowEnd; ++row) {
+        const TIn* xr = x + row * n2;
+        TOut* orow = out + row * n2;
+        Pack16<TIn> xv[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int v = j * kWave + lane;
+            if (v < nvec) xv[j] = loadPackStream(xr + v * EPV);
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int v = j * kWave + lane;
+            if (v < nvec) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const float f = toFloat(xv[j].e[e]);
+                    ss += f * f;
+                }
+            }
+        }
+        ss = waveSum(ss);
+        const float inv = 1.0f / sqrtf(ss * rn2 + eps);
+        if (lane == 0) invRms[row] = inv;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int v = j * kWave + lane;
+            if (v < nvec) {
+                TOut o[EPV];
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const TOut normed = fromFloat<TOut>(inv * toFloat(xv[j].e[e]));
+                    TOut r = fromFloat<TOut>(w[j][e] * toFloat(normed));
+                    if (HAS_BIAS) r = fromFloat<TOut>(toFloat(r) + b[j][e]);
+                    o[e] = r;
+                }
+                // EPV output elements are EPV*sizeof(TOut) contiguous bytes: 16, or 8 when fp32 -> 16-bit
+                if constexpr (sizeof(TOut) == sizeof(TIn)) {
+                    Pack16<TOut> pv;
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) pv.e[e] = o[e];
+                    storePackStream(orow + v * EPV, pv);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) orow[v * EPV + e] = o[e];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Forward, any shape / dtype combination: one wavefront per row, two sweeps over the row
+// (the second one hits in cache).  AccT is float or double.
+// ---------------------------------------------------------------------------
+template <typename TIn, typename TOut, typename AccT>
+__global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restrict__ out, AccT* __restrict__ invRms, const TIn* __restrict__ x,
+                                                                  const TOut* __restrict__ weight, const TOut* __restrict__ bias, int64_t n1, int64_t n2,
+                                                                  AccT eps) {
+    const int lane = threadIdx.x % kWave;
+    const int64_t wavesTotal = static_cast<int64_t>(gridDim.x) * kFwdWaves;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * kFwdWaves + threadIdx.x / kWave; row < n1; row += wavesTotal) {
+        const TIn* xr = x + row * n2;
+        TOut* orow = out + row * n2;
+        AccT ss = 0;
+        for (int64_t l = lane; l < n2; l += kWave) {
+            const AccT f = static_cast<AccT>(xr[l]);
+            ss += f * f;
+        }
+        ss = waveSum(ss);
+        AccT inv;
+        if constexpr (sizeof(AccT) == 8) {
+            inv = 1.0 / sqrt(ss / static_cast<AccT>(n2) + eps);
+        } else {
+            inv = 1.0f / sqrtf(ss / static_cast<AccT>(n2) + eps);
+        }
+        if (lane == 0) invRms[row] = inv;
+        for (int64_t l = lane; l < n2; l += kWave) {
+            const TOut normed = static_cast<TOut>(inv * static_cast<AccT>(xr[l]));
+            // the product of two OutT values is formed in the accumulation type and rounded once
+            TOut r = static_cast<TOut>(static_cast<AccT>(weight[l]) * static_cast<AccT>(normed));
+            if (bias != nullptr) r = static_cast<TOut>(static_cast<AccT>(r) + static_cast<AccT>(bias[l]));
+            orow[l] = r;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
+// Thread t of a 256-thread group owns packets t, t+256, ... of every row.
+// ---------------------------------------------------------------------------
+constexpr int kBwdThreads = 256;
+constexpr int kBwdWaves = kBwdThreads / kWave;
+
+template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS>
+__global__ __launch_bounds__(kBwdThreads) void rmsNormBwdFused(T* __restrict__ gradInput, ColAcc* __restrict__ partW, ColAcc* __restrict__ partB,
+                                                                const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
+                                                                const float* __restrict__ invRms, int64_t n1, int n2, int rowsPerBlock) {
+    constexpr int EPV = Pack16<T>::N;
+    __shared__ float red[2][kBwdWaves];
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int nvec = n2 / EPV;
+
+    float w[NVT][EPV];
+    ColAcc accW[NVT][EPV];
+    ColAcc accB[NVT][EPV];
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) {
+        const int v = j * kBwdThreads + tid;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            accW[j][e] = 0;
+            accB[j][e] = 0;
+            w[j][e] = (v < nvec) ? toFloat(weight[v * EPV + e]) : 0.f;
+        }
+    }
+
+    int64_t row = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
+    int64_t rowEnd = row + rowsPerBlock;
+    if (rowEnd > n1) rowEnd = n1;
+    const float fH = static_cast<float>(n2);
+    int parity = 0;
+    for (; row < rowEnd; ++row, parity ^= 1) {
+        const T* xr = x + row * n2;
+        const T* dr = dout + row * n2;
+        Pack16<T> xv[NVT], dv[NVT];
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kBwdThreads + tid;
+            if (v < nvec) {
+                xv[j] = loadPackStream(xr + v * EPV);
+                dv[j] = loadPackStream(dr + v * EPV);
+            }
+        }
+        const float inv = invRms[row];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kBwdThreads + tid;
+            if (v < nvec) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const float cx = toFloat(xv[j].e[e]);
+                    const float cd = toFloat(dv[j].e[e]);
+                    s += cd * w[j][e] * cx * inv;
+                    accW[j][e] += static_cast<ColAcc>(cd * cx * inv);
+                    if (HAS_GBIAS) accB[j][e] += static_cast<ColAcc>(cd);
+                }
+            }
+        }
+        s = waveSum(s);
+        if (lane == 0) red[parity][wave] = s;
+        __syncthreads();
+        float sum2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < kBwdWaves; ++i) sum2 += red[parity][i];
+        const float term1 = (1.0f / fH) * inv;
+        T* gr = gradInput + row * n2;
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kBwdThreads + tid;
+            if (v < nvec) {
+                Pack16<T> gv;
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const float cx = toFloat(xv[j].e[e]);
+                    const float cd = toFloat(dv[j].e[e]);
+                    float f = fH * cd * w[j][e];
+                    f -= cx * inv * sum2;
+                    f *= term1;
+                    gv.e[e] = fromFloat<T>(f);
+                }
+                storePackStream(gr + v * EPV, gv);
+            }
+        }
+    }
+
+    // this group's column partials
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) {
+        const int v = j * kBwdThreads + tid;
+        if (v < nvec) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                partW[static_cast<int64_t>(blockIdx.x) * n2 + v * EPV + e] = accW[j][e];
+                if (HAS_GBIAS) partB[static_cast<int64_t>(blockIdx.x) * n2 + v * EPV + e] = accB[j][e];
+            }
+        }
+    }
+}
+
+// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias).  A 256-thread group covers
+// 64 columns x 4 row slices; lanes of a wave read consecutive columns.
+template <typename T, typename ColAcc>
+__global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight, T* __restrict__ gradBias, const ColAcc* __restrict__ partW,
+                                                       const ColAcc* __restrict__ partB, int numParts, int n2) {
+    __shared__ double red[2][4][64];
+    const int lane = threadIdx.x % 64;
+    const int slice = threadIdx.x / 64;
+    const int col = blockIdx.x * 64 + lane;
+    double sw = 0.0, sb = 0.0;
+    if (col < n2) {
+        for (int p = slice; p < numParts; p += 4) {
+            sw += static_cast<double>(partW[static_cast<int64_t>(p) * n2 + col]);
+            if (gradBias != nullptr) sb += static_cast<double>(partB[static_cast<int64_t>(p) * n2 + col]);
+        }
+    }
+    red[0][slice][lane] = sw;
+    red[1][slice][lane] = sb;
+    __syncthreads();
+    if (slice == 0 && col < n2) {
+        sw = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
+        gradWeight[col] = fromDouble<T>(sw);
+        if (gradBias != nullptr) {
+            sb = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+            gradBias[col] = fromDouble<T>(sb);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, any shape / dtype combination (TX: x and grad_input; TV: dout, weight, grad_weight).
+// ---------------------------------------------------------------------------
+template <typename TX, typename TV, typename AccT>
+__global__ __launch_bounds__(kFwdThreads) void rmsNormBwdInputGeneric(TX* __restrict__ gradInput, const TV* __restrict__ dout, const TX* __restrict__ x,
+                                                                       const TV* __restrict__ weight, const AccT* __restrict__ invRms, int64_t n1,
+                                                                       int64_t n2) {
+    const int lane = threadIdx.x % kWave;
+    const int64_t wavesTotal = static_cast<int64_t>(gridDim.x) * kFwdWaves;
+    for (int64_t row = static_cast<int64_t>(blockIdx.x) * kFwdWaves + threadIdx.x / kWave; row < n1; row += wavesTotal) {
+        const TX* xr = x + row * n2;
+        const TV* dr = dout + row * n2;
+        const AccT inv = invRms[row];
+        AccT s = 0;
+        for (int64_t l = lane; l < n2; l += kWave) {
+            s += static_cast<AccT>(dr[l]) * static_cast<AccT>(weight[l]) * static_cast<AccT>(xr[l]) * inv;
+        }
+        s = waveSum(s);
+        const AccT fH = static_cast<AccT>(n2);
+        const AccT term1 = (static_cast<AccT>(1) / fH) * inv;
+        for (int64_t l = lane; l < n2; l += kWave) {
+            AccT f = fH * static_cast<AccT>(dr[l]) * static_cast<AccT>(weight[l]);
+            f -= static_cast<AccT>(xr[l]) * inv * s;
+            f *= term1;
+            gradInput[row * n2 + l] = static_cast<TX>(f);
+        }
+    }
+}
+
+// One thread per column, rows walked in order; the products are formed in AccT and summed in fp64.
+template <typename TX, typename TV, typename AccT>
+__global__ __launch_bounds__(256) void rmsNormBwdWeightGeneric(TV* __restrict__ gradWeight, TV* __restrict__ gradBias, const TV* __restrict__ dout,
+                                                                const TX* __restrict__ x, const AccT* __restrict__ invRms, int64_t n1, int64_t n2) {
+    const int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (col >= n2) return;
+    double sw = 0.0, sb = 0.0;
+    for (int64_t r = 0; r < n1; ++r) {
+        const AccT cd = static_cast<AccT>(dout[r * n2 + col]);
+        sw += static_cast<double>(cd * static_cast<AccT>(x[r * n2 + col]) * invRms[r]);
+        sb += static_cast<double>(cd);
+    }
+    gradWeight[col] = fromDouble<TV>(sw);
+    if (gradBias != nullptr) gradBias[col] = fromDouble<TV>(sb);
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+struct NormDims {
+    int64_t n1 = 1, n2 = 1;
+    int lead = 0;  // number of leading (non-normalised) dimensions
+};
+
+// Same rule as compute_n1_n2 / check_args in rmsnorm.cu:17-65 of the reference.
+diopiError_t normDims(const TensorView& input, diopiSize_t normalizedShape, NormDims* dims) {
+    ROCM_CHECK(normalizedShape.len >= 1 && normalizedShape.data != nullptr, "normalized_shape must have at least one dimension");
+    ROCM_CHECK(normalizedShape.len <= input.ndim, "normalized_shape has rank %lld but input has rank %d", static_cast<long long>(normalizedShape.len),
+               input.ndim);
+    dims->lead = input.ndim - static_cast<int>(normalizedShape.len);
+    dims->n1 = 1;
+    dims->n2 = 1;
+    for (int i = 0; i < dims->lead; ++i) dims->n1 *= input.shape[i];
+    for (int i = 0; i < normalizedShape.len; ++i) {
+        ROCM_CHECK(input.shape[dims->lead + i] == normalizedShape.data[i], "normalized_shape[%d] = %lld does not match input extent %lld", i,
+                   static_cast<long long>(normalizedShape.data[i]), static_cast<long long>(input.shape[dims->lead + i]));
+        dims->n2 *= normalizedShape.data[i];
+    }
+    return diopiSuccess;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// number of waves (or 256-thread groups) that are resident at once, used to size persistent launches
+int residentWavesTarget() { return deviceInfo().numCU * 12; }
+
+template <typename TIn, typename TOut>
+diopiError_t launchFwdFast(hipStream_t stream, const TensorView& out, const TensorView& invRms, const TensorView& in, const TensorView& w,
+                           const void* bias, const NormDims& d, double eps, bool* launched) {
+    constexpr int EPV = Pack16<TIn>::N;
+    *launched = false;
+    if (d.n2 % EPV != 0 || d.n2 > INT32_MAX) return diopiSuccess;
+    const int64_t nvec = d.n2 / EPV;
+    if (nvec > 16 * kWave) return diopiSuccess;
+    if (!aligned16(in.data) || !aligned16(out.data) || !aligned16(w.data)) return diopiSuccess;
+    if (sizeof(TOut) != sizeof(TIn) && (reinterpret_cast<uintptr_t>(out.data) & 7) != 0) return diopiSuccess;
+    const int nv = static_cast<int>(ceilDiv(nvec, kWave));
+    // every wave takes the same number of rows so that all of them fit on the device at once
+    int rowsPerWave = static_cast<int>(ceilDiv(d.n1, residentWavesTarget()));
+    if (rowsPerWave < 1) rowsPerWave = 1;
+    const int64_t waves = ceilDiv(d.n1, rowsPerWave);
+    const unsigned grid = static_cast<unsigned>(ceilDiv(waves, kFwdWaves));
+    const float feps = static_cast<float>(eps);
+    const int n2 = static_cast<int>(d.n2);
+#define ROCM_FWD_CASE(NVC)                                                                                                                          \
+    if (bias != nullptr) {                                                                                                                          \
+        hipLaunchKernelGGL((rmsNormFwdRowReg<TIn, TOut, NVC, true>), dim3(grid), dim3(kFwdThreads), 0, stream, static_cast<TOut*>(out.data),         \
+                           static_cast<float*>(invRms.data), static_cast<const TIn*>(in.data), static_cast<const TOut*>(w.data),                      \
+                           static_cast<const TOut*>(bias), d.n1, n2, feps, rowsPerWave);                                                              \
+    } else {                                                                                                                                        \
+        hipLaunchKernelGGL((rmsNormFwdRowReg<TIn, TOut, NVC, false>), dim3(grid), dim3(kFwdThreads), 0, stream, static_cast<TOut*>(out.data),        \
+                           static_cast<float*>(invRms.data), static_cast<const TIn*>(in.data), static_cast<const TOut*>(w.data),                      \
+                           static_cast<const TOut*>(nullptr), d.n1, n2, feps, rowsPerWave);                                                           \
+    }
+    if (nv <= 1) {
+        ROCM_FWD_CASE(1)
+    } else if (nv <= 2) {
+        ROCM_FWD_CASE(2)
+    } else if (nv <= 4) {
+        ROCM_FWD_CASE(4)
+    } else if (nv <= 8) {
+        ROCM_FWD_CASE(8)
+    } else {
+        ROCM_FWD_CASE(16)
+    }
+#undef ROCM_FWD_CASE
+    ROCM_LAUNCH_CHECK();
+    *launched = true;
+    return diopiSuccess;
+}
+
+template <typename TIn, typename TOut, typename AccT>
+diopiError_t launchFwdGeneric(hipStream_t stream, const TensorView& out, const TensorView& invRms, const TensorView& in, const TensorView& w,
+                              const void* bias, const NormDims& d, double eps) {
+    int64_t blocks = ceilDiv(d.n1, kFwdWaves);
+    const int64_t cap = static_cast<int64_t>(deviceInfo().numCU) * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((rmsNormFwdGeneric<TIn, TOut, AccT>), dim3(static_cast<unsigned>(blocks)), dim3(kFwdThreads), 0, stream,
+                       static_cast<TOut*>(out.data), static_cast<AccT*>(invRms.data), static_cast<const TIn*>(in.data), static_cast<const TOut*>(w.data),
+                       static_cast<const TOut*>(bias), d.n1, d.n2, static_cast<AccT>(eps));
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
+template <typename TIn, typename TOut>
+diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const TensorView& invRms, const TensorView& in, const TensorView& w,
+                          const void* bias, const NormDims& d, double eps) {
+    using AccT = typename AccType<TIn>::type;
+    if constexpr (sizeof(AccT) == 4 && sizeof(TIn) >= sizeof(TOut)) {
+        bool launched = false;
+        ROCM_CALL((launchFwdFast<TIn, TOut>(stream, out, invRms, in, w, bias, d, eps, &launched)));
+        if (launched) return diopiSuccess;
+    }
+    return launchFwdGeneric<TIn, TOut, AccT>(stream, out, invRms, in, w, bias, d, eps);
+}
+
+template <typename T, typename ColAcc>
+diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& gIn, const TensorView& gW, void* gBias, const TensorView& dout,
+                            const TensorView& in, const TensorView& w, const TensorView& invRms, const NormDims& d, bool* launched) {
+    constexpr int EPV = Pack16<T>::N;
+    *launched = false;
+    if (d.n2 % EPV != 0 || d.n2 > INT32_MAX) return diopiSuccess;
+    const int64_t nvec = d.n2 / EPV;
+    if (nvec > 4 * kBwdThreads) return diopiSuccess;
+    if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
+    const int nvt = static_cast<int>(ceilDiv(nvec, kBwdThreads));
+    int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * envInt("DIOPI_ROCM_RMSBWD_BLOCKS_PER_CU", 4);
+    int rowsPerBlock = static_cast<int>(ceilDiv(d.n1, maxBlocks));
+    if (rowsPerBlock < 1) rowsPerBlock = 1;
+    const int numParts = static_cast<int>(ceilDiv(d.n1, rowsPerBlock));
+    const int n2 = static_cast<int>(d.n2);
+    const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(ColAcc);
+    void* scratch = nullptr;
+    ROCM_CALL(requireScratch(ctx, partBytes * (gBias ? 2 : 1), &scratch));
+    ColAcc* partW = static_cast<ColAcc*>(scratch);
+    ColAcc* partB = gBias ? partW + static_cast<int64_t>(numParts) * n2 : nullptr;
+#define ROCM_BWD_CASE(NVC)                                                                                                                             \
+    if (gBias != nullptr) {                                                                                                                            \
+        hipLaunchKernelGGL((rmsNormBwdFused<T, ColAcc, NVC, true>), dim3(numParts), dim3(kBwdThreads), 0, stream, static_cast<T*>(gIn.data), partW,     \
+                           partB, static_cast<const T*>(dout.data), static_cast<const T*>(in.data), static_cast<const T*>(w.data),                      \
+                           static_cast<const float*>(invRms.data), d.n1, n2, rowsPerBlock);                                                             \
+    } else {                                                                                                                                           \
+        hipLaunchKernelGGL((rmsNormBwdFused<T, ColAcc, NVC, false>), dim3(numParts), dim3(kBwdThreads), 0, stream, static_cast<T*>(gIn.data), partW,    \
+                           partB, static_cast<const T*>(dout.data), static_cast<const T*>(in.data), static_cast<const T*>(w.data),                      \
+                           static_cast<const float*>(invRms.data), d.n1, n2, rowsPerBlock);                                                             \
+    }
+    if (nvt <= 1) {
+        ROCM_BWD_CASE(1)
+    } else if (nvt <= 2) {
+        ROCM_BWD_CASE(2)
+    } else {
+        ROCM_BWD_CASE(4)
+    }
+#undef ROCM_BWD_CASE
+    ROCM_LAUNCH_CHECK();
+    hipLaunchKernelGGL((rmsNormBwdFold<T, ColAcc>), dim3(static_cast<unsigned>(ceilDiv(n2, 64))), dim3(256), 0, stream, static_cast<T*>(gW.data),
+                       static_cast<T*>(gBias), partW, partB, numParts, n2);
+    ROCM_LAUNCH_CHECK();
+    *launched = true;
+    return diopiSuccess;
+}
+
+template <typename TX, typename TV>
+diopiError_t backwardTyped(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& gIn, const TensorView& gW, void* gBias, const TensorView& dout,
+                           const TensorView& in, const TensorView& w, const TensorView& invRms, const NormDims& d) {
+    using AccT = typename AccType<TX>::type;
+    if constexpr (std::is_same<TX, TV>::value && sizeof(AccT) == 4) {
+        bool launched = false;
+        if constexpr (sizeof(TX) == 4) {
+            ROCM_CALL((launchBwdFused<TX, double>(ctx, stream, gIn, gW, gBias, dout, in, w, invRms, d, &launched)));
+        } else {
+            ROCM_CALL((launchBwdFused<TX, float>(ctx, stream, gIn, gW, gBias, dout, in, w, invRms, d, &launched)));
+        }
+        if (launched) return diopiSuccess;
+    }
+    int64_t blocks = ceilDiv(d.n1, kFwdWaves);
+    const int64_t cap = static_cast<int64_t>(deviceInfo().numCU) * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((rmsNormBwdInputGeneric<TX, TV, AccT>), dim3(static_cast<unsigned>(blocks)), dim3(kFwdThreads), 0, stream,
+                       static_cast<TX*>(gIn.data), static_cast<const TV*>(dout.data), static_cast<const TX*>(in.data), static_cast<const TV*>(w.data),
+                       static_cast<const AccT*>(invRms.data), d.n1, d.n2);
+    ROCM_LAUNCH_CHECK();
+    hipLaunchKernelGGL((rmsNormBwdWeightGeneric<TX, TV, AccT>), dim3(static_cast<unsigned>(ceilDiv(d.n2, 256))), dim3(256), 0, stream,
+                       static_cast<TV*>(gW.data), static_cast<TV*>(gBias), static_cast<const TV*>(dout.data), static_cast<const TX*>(in.data),
+                       static_cast<const AccT*>(invRms.data), d.n1, d.n2);
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
+// inv_rms carries the leading dimensions of the input (diopi_functions.py:7046-7054 of the reference).
+diopiError_t checkInvRms(const TensorView& invRms, const TensorView& in, const NormDims& d) {
+    const diopiDtype_t want = in.dtype == diopi_dtype_float64 ? diopi_dtype_float64 : diopi_dtype_float32;
+    ROCM_CHECK(invRms.dtype == want, "inv_rms must be %s for %s input, got %s", dtypeName(want), dtypeName(in.dtype), dtypeName(invRms.dtype));
+    ROCM_CHECK(invRms.numel == d.n1, "inv_rms has %lld elements, expected %lld (the leading dimensions of input)", static_cast<long long>(invRms.numel),
+               static_cast<long long>(d.n1));
+    return diopiSuccess;
+}
+
+diopiError_t checkParam(const TensorView& p, const char* name, diopiSize_t normalizedShape, diopiDtype_t dtype) {
+    ROCM_CHECK(p.dtype == dtype, "%s must have dtype %s, got %s", name, dtypeName(dtype), dtypeName(p.dtype));
+    ROCM_CHECK(p.ndim == normalizedShape.len, "%s must have the shape of normalized_shape", name);
+    for (int i = 0; i < p.ndim; ++i) {
+        ROCM_CHECK(p.shape[i] == normalizedShape.data[i], "%s must have the shape of normalized_shape", name);
+    }
+    return diopiSuccess;
+}
+
+}  // namespace
+}  // namespace rocm
+
+extern "C" diopiError_t diopiRMSNorm(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiTensorHandle_t inv_rms, diopiConstTensorHandle_t input,
+                                     diopiSize_t normalized_shape, diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias, double eps) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    TensorView vOut, vInv, vIn, vW, vB;
+    ROCM_CALL(unwrap(out, "out", &vOut));
+    ROCM_CALL(unwrap(inv_rms, "inv_rms", &vInv));
+    ROCM_CALL(unwrap(input, "input", &vIn));
+    ROCM_CALL(unwrap(weight, "weight", &vW));
+    ROCM_CALL(requireDeviceContiguous(vOut, "out"));
+    ROCM_CALL(requireDeviceContiguous(vInv, "inv_rms"));
+    ROCM_CALL(requireDeviceContiguous(vIn, "input"));
+    ROCM_CALL(requireDeviceContiguous(vW, "weight"));
+    if (bias != nullptr) {
+        ROCM_CALL(unwrap(bias, "bias", &vB));
+        ROCM_CALL(requireDeviceContiguous(vB, "bias"));
+    }
+    NormDims d;
+    ROCM_CALL(normDims(vIn, normalized_shape, &d));
+    ROCM_CHECK(vOut.sameShape(vIn), "out must have the shape of input");
+    ROCM_CHECK(isFloatDtype(vIn.dtype) && isFloatDtype(vOut.dtype), "input/out dtypes %s/%s are not supported", dtypeName(vIn.dtype),
+               dtypeName(vOut.dtype));
+    ROCM_CALL(checkParam(vW, "weight", normalized_shape, vOut.dtype));
+    if (bias != nullptr) ROCM_CALL(checkParam(vB, "bias", normalized_shape, vOut.dtype));
+    ROCM_CALL(checkInvRms(vInv, vIn, d));
+    if (vIn.numel == 0) return diopiSuccess;
+
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    const void* pb = bias ? vB.data : nullptr;
+    // accepted (input, out) dtype pairs: layer_norm_cuda_kernel.cu:841-908 of the reference
+    const diopiDtype_t ti = vIn.dtype, to = vOut.dtype;
+    if (ti == diopi_dtype_float32 && to == diopi_dtype_float32) return forwardTyped<float, float>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float16 && to == diopi_dtype_float16) return forwardTyped<half_t, half_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_bfloat16 && to == diopi_dtype_bfloat16) return forwardTyped<bf16_t, bf16_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float32 && to == diopi_dtype_float16) return forwardTyped<float, half_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float32 && to == diopi_dtype_bfloat16) return forwardTyped<float, bf16_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float64 && to == diopi_dtype_float64) return forwardTyped<double, double>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float64 && to == diopi_dtype_float32) return forwardTyped<double, float>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float64 && to == diopi_dtype_float16) return forwardTyped<double, half_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    if (ti == diopi_dtype_float64 && to == diopi_dtype_bfloat16) return forwardTyped<double, bf16_t>(stream, vOut, vInv, vIn, vW, pb, d, eps);
+    setLastError("diopiRMSNorm: input dtype %s with out dtype %s is not supported", dtypeName(ti), dtypeName(to));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}
+
+extern "C" diopiError_t diopiRMSNormBackward(diopiContextHandle_t ctx, diopiTensorHandle_t grad_input, diopiTensorHandle_t grad_weight,
+                                             diopiTensorHandle_t grad_bias, diopiConstTensorHandle_t grad_output, diopiConstTensorHandle_t input,
+                                             diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias, diopiConstTensorHandle_t inv_rms,
+                                             diopiSize_t normalized_shape, double eps) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)bias;  // the reference ignores both (functions_ext.cpp:82-107)
+    (void)eps;
+    TensorView vGI, vGW, vGB, vDo, vIn, vW, vInv;
+    ROCM_CALL(unwrap(grad_input, "grad_input", &vGI));
+    ROCM_CALL(unwrap(grad_weight, "grad_weight", &vGW));
+    ROCM_CALL(unwrap(grad_output, "grad_output", &vDo));
+    ROCM_CALL(unwrap(input, "input", &vIn));
+    ROCM_CALL(unwrap(weight, "weight", &vW));
+    ROCM_CALL(unwrap(inv_rms, "inv_rms", &vInv));
+    ROCM_CALL(requireDeviceContiguous(vGI, "grad_input"));
+    ROCM_CALL(requireDeviceContiguous(vGW, "grad_weight"));
+    ROCM_CALL(requireDeviceContiguous(vDo, "grad_output"));
+    ROCM_CALL(requireDeviceContiguous(vIn, "input"));
+    ROCM_CALL(requireDeviceContiguous(vW, "weight"));
+    ROCM_CALL(requireDeviceContiguous(vInv, "inv_rms"));
+    if (grad_bias != nullptr) {
+        ROCM_CALL(unwrap(grad_bias, "grad_bias", &vGB));
+        ROCM_CALL(requireDeviceContiguous(vGB, "grad_bias"));
+    }
+    NormDims d;
+    ROCM_CALL(normDims(vIn, normalized_shape, &d));
+    ROCM_CHECK(vGI.sameShape(vIn) && vGI.dtype == vIn.dtype, "grad_input must have the shape and dtype of input");
+    ROCM_CHECK(vDo.sameShape(vIn), "grad_output must have the shape of input");
+    ROCM_CHECK(isFloatDtype(vIn.dtype) && isFloatDtype(vW.dtype), "input/weight dtypes %s/%s are not supported", dtypeName(vIn.dtype),
+               dtypeName(vW.dtype));
+    ROCM_CALL(checkParam(vW, "weight", normalized_shape, vW.dtype));
+    ROCM_CHECK(vDo.dtype == vW.dtype, "grad_output must have the dtype of weight (%s), got %s", dtypeName(vW.dtype), dtypeName(vDo.dtype));
+    ROCM_CALL(checkParam(vGW, "grad_weight", normalized_shape, vW.dtype));
+    if (grad_bias != nullptr) ROCM_CALL(checkParam(vGB, "grad_bias", normalized_shape, vW.dtype));
+    ROCM_CALL(checkInvRms(vInv, vIn, d));
+    if (d.n2 == 0) return diopiSuccess;
+
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    void* pgb = grad_bias ? vGB.data : nullptr;
+    if (d.n1 == 0) {
+        // no rows: the column sums are empty sums
+        ROCM_CALL(zeroFill(stream, vGW.data, vGW.nbytes()));
+        if (pgb) ROCM_CALL(zeroFill(stream, pgb, vGB.nbytes()));
+        return diopiSuccess;
+    }
+    const diopiDtype_t tx = vIn.dtype, tv = vW.dtype;
+    if (tx == diopi_dtype_float32 && tv == diopi_dtype_float32) return backwardTyped<float, float>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    if (tx == diopi_dtype_float16 && tv == diopi_dtype_float16) return backwardTyped<half_t, half_t>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    if (tx == diopi_dtype_bfloat16 && tv == diopi_dtype_bfloat16)
+        return backwardTyped<bf16_t, bf16_t>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    if (tx == diopi_dtype_float32 && tv == diopi_dtype_float16) return backwardTyped<float, half_t>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    if (tx == diopi_dtype_float32 && tv == diopi_dtype_bfloat16) return backwardTyped<float, bf16_t>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    if (tx == diopi_dtype_float64 && tv == diopi_dtype_float64) return backwardTyped<double, double>(ctx, stream, vGI, vGW, pgb, vDo, vIn, vW, vInv, d);
+    setLastError("diopiRMSNormBackward: input dtype %s with weight dtype %s is not supported", dtypeName(tx), dtypeName(tv));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}

@@ -1,0 +1,144 @@
+"""Python callers of the seven LLaMA-inference operators, through the C ABI.
+
+Each function mirrors the wrapper of the same name in
+``diopi_test/python/conformance/diopi_functions.py`` of the reference
+(rotary_emb 7030-7037, rms_norm 7040-7070, rms_norm_backward 7073-7109,
+destindex_copy_kv 7896-7902, token_attention 7905-7911,
+token_softmax_reducev 7914-7939, context_attention 7942-7948): same argument
+order and meaning, outputs allocated by the caller side with the reference's
+shape/dtype rules, return code checked with the reference's policy.
+
+Arguments are torch tensors on the GPU; they are wrapped as diopiTensor handles
+for the duration of the call.  The operators run on the context's stream; the
+wrappers order that stream after torch's current stream on entry and torch's
+current stream after it on exit, so results can be used by torch code directly.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from . import runtime as rt
+from .runtime import Sizes, Tensor, as_handle, check_returncode
+
+# inv_rms of the last rms_norm call, consumed by rms_norm_backward
+# (reference: GLOBAL_STATE["rms_norm_inv_rms"], diopi_functions.py:7069, 7087)
+GLOBAL_STATE = {}
+
+
+def _ctx(ctx: Optional[rt.Context]) -> rt.Context:
+    return ctx if ctx is not None else rt.default_context()
+
+
+class _on_stream:
+    """Orders the context's stream with torch's current stream around a call."""
+
+    def __init__(self, ctx: rt.Context, *tensors):
+        self.ctx = ctx
+        self.cuda = ctx.torch_stream is not None and any(t is not None and t.is_cuda for t in tensors)
+
+    def __enter__(self):
+        if self.cuda:
+            self.ctx.torch_stream.wait_stream(torch.cuda.current_stream())
+        return self
+
+    def __exit__(self, *exc):
+        if self.cuda:
+            torch.cuda.current_stream().wait_stream(self.ctx.torch_stream)
+        return False
+
+
+def _handles(*tensors):
+    """Wraps torch tensors as diopiTensor handles.  Returns (keepalive, handles): the wrappers own the
+    handles, so `keepalive` must stay referenced until the call has returned."""
+    keep = [None if t is None else Tensor(t) for t in tensors]
+    return keep, [as_handle(k) for k in keep]
+
+
+def rotary_emb(input: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, conj: bool, interleaved: bool, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    out = torch.empty_like(input, memory_format=torch.contiguous_format)
+    with _on_stream(ctx, input):
+        keep, h = _handles(out, input, cos, sin)
+        ret = rt.libs().impl.diopiRotaryEmbedding(ctx.handle, *h, bool(conj), bool(interleaved))
+    check_returncode(ret, "diopiRotaryEmbedding")
+    return out
+
+
+def rms_norm(input: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+             ctx: Optional[rt.Context] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    out = torch.empty(input.shape, dtype=out_dtype or input.dtype, device=input.device)
+    n = len(normalized_shape)
+    inv_shape = list(input.shape)[: input.dim() - n]
+    # 16-bit and fp32 inputs keep their statistics in fp32, fp64 inputs in fp64
+    inv_dtype = torch.float64 if input.dtype == torch.float64 else torch.float32
+    inv_rms = torch.empty(inv_shape, dtype=inv_dtype, device=input.device)
+    sizes = Sizes(normalized_shape)
+    with _on_stream(ctx, input):
+        keep, h = _handles(out, inv_rms, input, weight, bias)
+        ret = rt.libs().impl.diopiRMSNorm(ctx.handle, h[0], h[1], h[2], sizes.c, h[3], h[4], float(eps))
+    check_returncode(ret, "diopiRMSNorm")
+    GLOBAL_STATE["rms_norm_inv_rms"] = inv_rms
+    return out
+
+
+def rms_norm_backward(grad_outputs: Sequence[torch.Tensor], input: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor],
+                      normalized_shape: Sequence[int], eps: float, ctx: Optional[rt.Context] = None, inv_rms: Optional[torch.Tensor] = None) -> dict:
+    ctx = _ctx(ctx)
+    grad_input = torch.empty_like(input)
+    grad_weight = torch.empty_like(weight)
+    grad_bias = torch.empty_like(bias) if bias is not None else None
+    if inv_rms is None:
+        inv_rms = GLOBAL_STATE.pop("rms_norm_inv_rms")
+    sizes = Sizes(normalized_shape)
+    with _on_stream(ctx, input):
+        keep, h = _handles(grad_input, grad_weight, grad_bias, grad_outputs[0], input, weight, bias, inv_rms)
+        ret = rt.libs().impl.diopiRMSNormBackward(ctx.handle, *h, sizes.c, float(eps))
+    ctx.clear_tensors()
+    check_returncode(ret, "diopiRMSNormBackward")
+    out = {"input": grad_input, "weight": grad_weight}
+    if bias is not None:
+        out["bias"] = grad_bias
+    return out
+
+
+def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, k, dest_loc)
+        ret = rt.libs().impl.diopiDestIndexCopyKV(ctx.handle, *h)
+    check_returncode(ret, "diopiDestIndexCopyKV")
+    return out
+
+
+def token_attention(q: torch.Tensor, k: torch.Tensor, out: torch.Tensor, b_loc: torch.Tensor, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor,
+                    max_input_len: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, q, k, b_loc, b_start_loc, b_seq_len)
+        ret = rt.libs().impl.diopiTokenAttentionInference(ctx.handle, *h, int(max_input_len))
+    check_returncode(ret, "diopiTokenAttentionInference")
+    return out
+
+
+def token_softmax_reducev(logics: torch.Tensor, v: torch.Tensor, out: torch.Tensor, b_loc: torch.Tensor, b_start_loc: torch.Tensor,
+                          b_seq_len: torch.Tensor, max_input_len: int, other_kv_index: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, logics, v, b_loc, b_start_loc, b_seq_len)
+        ret = rt.libs().impl.diopiTokenSoftmaxReduceVInference(ctx.handle, *h, int(max_input_len), int(other_kv_index))
+    ctx.clear_tensors()
+    check_returncode(ret, "diopiTokenSoftmaxReduceVInference")
+    return out
+
+
+def context_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor,
+                      max_input_len: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, q, k, v, b_start_loc, b_seq_len)
+        ret = rt.libs().impl.diopiContextAttentionInference(ctx.handle, *h, int(max_input_len))
+    check_returncode(ret, "diopiContextAttentionInference")
+    return out

@@ -1,0 +1,113 @@
+/*
+ * The LLaMA-inference operator family of the DIOPI extension ABI, as exported
+ * by the gfx950 build of libdiopi_impl.so.  Signatures restate
+ * proto/include/diopi/functions_ext.h of the reference (line numbers cited at
+ * each prototype) and must stay declaration-compatible with it.
+ *
+ * Common rules for every operator here:
+ *  - all tensors live on the device, are contiguous, and are allocated by the
+ *    caller (outputs included); optional tensors are passed as NULL;
+ *  - work is enqueued on the stream of `ctx` and the call returns without
+ *    waiting for it;
+ *  - index tensors (dest_loc, b_loc, b_start_loc, b_seq_len) may be int32 or
+ *    int64 and are read on the device only: no host synchronisation;
+ *  - the return value is a diopiError_t; on failure the text is available
+ *    from diopiGetLastErrorString().
+ */
+#ifndef DIOPI_ROCM_INCLUDE_DIOPI_FUNCTIONS_EXT_H_
+#define DIOPI_ROCM_INCLUDE_DIOPI_FUNCTIONS_EXT_H_
+
+#include <diopi/diopirt.h>
+#include <stdbool.h>
+#include <stdint.h>
+
+#if defined(__cplusplus)
+extern "C" {
+#endif
+
+/*
+ * Rotary position embedding on the two halves of the last dimension.
+ * reference: functions_ext.h:31-32.
+ *   x1 = x[..., :D/2], x2 = x[..., D/2:]; cos/sin broadcast (right-aligned) against x1.
+ *   conj == false: out1 = x1*cos - x2*sin, out2 = x1*sin + x2*cos
+ *   conj == true : out1 = x1*cos + x2*sin, out2 = -x1*sin + x2*cos
+ * Arithmetic is fp32 with one rounding to the element type (fp64 inputs too).
+ * interleaved == true returns diopiNoImplement, as the reference does.
+ * dtypes: float16, bfloat16, float32, float64 (out, x, cos, sin share one dtype).
+ */
+DIOPI_API diopiError_t diopiRotaryEmbedding(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t x, diopiConstTensorHandle_t cos,
+                                            diopiConstTensorHandle_t sin, const bool conj, const bool interleaved);
+
+/*
+ * RMS normalisation over the trailing `normalized_shape` dimensions.
+ * reference: functions_ext.h:45-46.
+ *   inv_rms[row] = rsqrt(mean(x[row]^2) + eps)         (fp32 accumulate; fp64 for fp64 input)
+ *   out[row]     = weight * round_to_out_dtype(inv_rms[row] * x[row])  (+ bias if bias != NULL)
+ * inv_rms has the leading dimensions of input and dtype float32 (float64 for float64 input).
+ * out/weight/bias share one dtype; input may be the same dtype, or float32 with a 16-bit out.
+ */
+DIOPI_API diopiError_t diopiRMSNorm(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiTensorHandle_t inv_rms, diopiConstTensorHandle_t input,
+                                    diopiSize_t normalized_shape, diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias, double eps);
+
+/*
+ * Gradient of diopiRMSNorm.  reference: functions_ext.h:62-65.
+ *   g = grad_output * weight;  s = sum_l g_l * x_l * inv_rms          (per row)
+ *   grad_input_l  = (inv_rms / n2) * (n2 * g_l - x_l * inv_rms * s)
+ *   grad_weight_j = sum_rows grad_output * x * inv_rms
+ *   grad_bias     = grad_output summed over the leading dimensions (only if grad_bias != NULL)
+ * `bias` and `eps` are accepted and unused, as in the reference.  Needs one
+ * scratch buffer from diopiRequireBuffer for the partial column sums.
+ */
+DIOPI_API diopiError_t diopiRMSNormBackward(diopiContextHandle_t ctx, diopiTensorHandle_t grad_input, diopiTensorHandle_t grad_weight,
+                                            diopiTensorHandle_t grad_bias, diopiConstTensorHandle_t grad_output, diopiConstTensorHandle_t input,
+                                            diopiConstTensorHandle_t weight, diopiConstTensorHandle_t bias, diopiConstTensorHandle_t inv_rms,
+                                            diopiSize_t normalized_shape, double eps);
+
+/*
+ * KV-cache row scatter: out[dest_loc[t], :, :] = k[t, :, :].  reference: functions_ext.h:563.
+ * Bit-exact copy, no dtype conversion; rows of `out` not named by dest_loc are
+ * untouched.  Negative indices wrap once (index + rows); indices still out of
+ * range are skipped.  Duplicate indices: one of the rows wins, unspecified which.
+ */
+DIOPI_API diopiError_t diopiDestIndexCopyKV(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t k, diopiConstTensorHandle_t dest_loc);
+
+/*
+ * Decode attention, first half: scaled q.k for every cached token of every sequence.
+ * reference: functions_ext.h:579-581.
+ *   slots_i = b_loc[i, max_input_len - L_i : max_input_len]           (right-aligned window)
+ *   token_attention_out[h, b_start_loc[i] + t] = dot(q[i, h, :], k[slots_i[t], h / G, :]) / sqrt(D)
+ * q [B, H, D]; k [slots, Hkv, D] with H = G * Hkv (G = 1 is the reference's case);
+ * out [H, sum L].  Columns not covered by any sequence are left untouched.
+ */
+DIOPI_API diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t token_attention_out, diopiConstTensorHandle_t q,
+                                                    diopiConstTensorHandle_t k, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
+                                                    diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+/*
+ * Decode attention, second half: softmax over each sequence's logits, then the weighted sum of V.
+ * reference: functions_ext.h:597-599.
+ *   P = softmax(logics[h, b_start_loc[i] : b_start_loc[i] + L_i])     (fp32 inside)
+ *   out[i, h, :] = sum_t P[t] * v[slots_i[t], h / G, :]
+ * other_kv_index is accepted and ignored, as in the reference.  Needs scratch from
+ * diopiRequireBuffer when a sequence is split over several work-groups.
+ */
+DIOPI_API diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t logics,
+                                                         diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
+                                                         diopiConstTensorHandle_t b_seq_len, int max_input_len, int other_kv_index);
+
+/*
+ * Prefill attention: causal softmax(q k^T / sqrt(D)) v per packed sequence.
+ * reference: functions_ext.h:634-636.
+ * q, k, v, out [sum L, H, D]; sequence i owns rows [b_start_loc[i], b_start_loc[i] + b_seq_len[i]).
+ * Rows outside every sequence are left untouched.  max_input_len is only an upper
+ * bound used to size the launch (the reference never reads it).
+ */
+DIOPI_API diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
+                                                      diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
+                                                      diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+#if defined(__cplusplus)
+}
+#endif
+
+#endif /* DIOPI_ROCM_INCLUDE_DIOPI_FUNCTIONS_EXT_H_ */

@@ -1,0 +1,222 @@
+"""CPU oracle for the seven LLaMA-inference operators.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, on the CPU with plain ATen (torch) and numpy calls, what the reference
+computes for each operator.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
+leg of ``bench.py`` may import it, and only as the checker; the product never routes through it.
+
+Each function follows the reference line by line (citations are relative to the reference tree):
+
+===========================  =====================================================================
+rms_norm                     impl/torch/functions/functions_ext.cpp:66-80,
+                             functions_ext/layer_norm_cuda_kernel.cu:321-366 (cuApplyRMSNorm),
+                             functions_ext/rmsnorm.cu:17-28; Python twin customized_test.py:392-403
+rms_norm_backward            functions_ext.cpp:82-107, layer_norm_cuda_kernel.cu:402, 444, 572-717
+rotary_emb                   functions_ext.cpp:43-64, functions_ext/rotary.cu:26-44;
+                             customized_test.py:374-390
+destindex_copy_kv            functions_lightllm.cpp:18-26; customized_test.py:694-696
+token_attention              functions_lightllm.cpp:53-80; customized_test.py:698-713
+token_softmax_reducev        functions_lightllm.cpp:82-107; customized_test.py:715-733
+context_attention            functions_lightllm.cpp:109-147; customized_test.py:8-33, 735-749
+===========================  =====================================================================
+
+Two arithmetic modes:
+
+* ``exact=False`` keeps every intermediate in the dtype the reference keeps it in (16-bit matmul
+  results rounded to 16 bits, fp32 softmax, probabilities rounded back, ...), i.e. it is the
+  reference's composition run by ATen on the CPU.  This is also what ``bench.py`` times as the CPU
+  baseline.
+* ``exact=True`` evaluates the same mathematical expression in float64 from the same inputs and
+  rounds once at the end: the reference point for "how far from the true value" reports.
+
+Grouped-query attention (H = G * Hkv query heads over Hkv cache heads) is an extension of the two
+decode operators: query head h reads cache head h // G (the grouping rule of the reference's
+flash-attention test, customized_test.py:466-472).  With G == 1 the functions are the reference's.
+
+How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"):
+  rms_norm / backward  closed forms (constant rows, +-1 rows, scale invariance, sum((out/w)^2)),
+                       float64 autograd of the textbook formula, the identity
+                       sum_l x_l*grad_input_l = eps*inv_rms^3*sum_l g_l*x_l, column sums in float64
+  rotary_emb           position 0 is the identity bit for bit, norm preservation per pair,
+                       conj undoes the rotation, the reference's broadcasting shapes
+                       (diopi_configs.py:9066-9074), empty tensors (9093)
+  destindex_copy_kv    the reference fixtures dest_loc=(0..4),(14..17) into 120 rows
+                       (diopi_configs.py:9321-9333), untouched rows compared byte for byte
+  token_attention      the reference's integer fixture (diopi_configs.py:9541-9558) read against an
+                       independent statement of the window: sequence 0 reads slots [0,1,2,10],
+                       1 reads [3,4,5,6,11], 2 reads [7,8,9,12]; L=1 and k=q closed forms; float64
+                       brute force with explicit Python loops
+  token_softmax_reducev  constant logits -> mean of the gathered rows, one dominant logit -> that row,
+                       L=1 -> the row bit for bit, float64 brute force
+  context_attention    first token of every sequence returns its v row bit for bit, constant V,
+                       the reference's ragged fixtures (diopi_configs.py:9349-9377) incl. untouched
+                       rows, float64 brute force, and the last row cross-checked against
+                       token_attention + token_softmax_reducev on the same K/V
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+def _n1_n2(shape: Sequence[int], normalized_shape: Sequence[int]) -> Tuple[int, int]:
+    """rmsnorm.cu:17-28 (compute_n1_n2): n2 = prod(normalized_shape), n1 = product of the leading dims."""
+    nd = len(normalized_shape)
+    assert nd >= 1 and tuple(shape[len(shape) - nd:]) == tuple(normalized_shape), "normalized_shape must match the trailing dims"
+    n2 = int(np.prod(normalized_shape)) if nd else 1
+    n1 = int(np.prod(shape[: len(shape) - nd])) if len(shape) > nd else 1
+    return n1, n2
+
+
+def rms_norm(input: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+             exact: bool = False, out_dtype: Optional[torch.dtype] = None):
+    """Returns (out, inv_rms).  inv_rms has the leading dims of input, fp32 (fp64 for fp64 input)."""
+    out_dtype = out_dtype or input.dtype
+    n1, n2 = _n1_n2(input.shape, normalized_shape)
+    lead = list(input.shape[: input.dim() - len(normalized_shape)])
+    if exact:
+        x = input.double().reshape(n1, n2)
+        inv = 1.0 / torch.sqrt((x * x).sum(-1, keepdim=True) / n2 + eps)
+        out = weight.double().reshape(1, n2) * (inv * x)
+        if bias is not None:
+            out = out + bias.double().reshape(1, n2)
+        return out.reshape(input.shape), inv.reshape(lead)
+    acc = torch.float64 if input.dtype == torch.float64 else torch.float32  # at::acc_type, kernel.cu:971
+    x = input.to(acc).reshape(n1, n2)
+    sigma2 = (x * x).sum(-1, keepdim=True) / n2  # cuWelfordMuSigma2 with rms_only, then / n2
+    inv = torch.rsqrt(sigma2 + torch.tensor(eps, dtype=acc))  # kernel.cu:336, eps cast to U at 742
+    normed = (inv * x).to(out_dtype)  # static_cast<V>(c_invvar * curr), kernel.cu:345
+    out = weight.reshape(1, n2) * normed  # V * V, rounded to V
+    if bias is not None:
+        out = out + bias.reshape(1, n2)  # atOut.add_(atBias), functions_ext.cpp:75-78
+    return out.reshape(input.shape), inv.reshape(lead)
+
+
+def rms_norm_backward(grad_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor, inv_rms: torch.Tensor,
+                      normalized_shape: Sequence[int], with_bias: bool = False, exact: bool = False):
+    """Returns (grad_input, grad_weight, grad_bias-or-None)."""
+    n1, n2 = _n1_n2(input.shape, normalized_shape)
+    acc = torch.float64 if (exact or input.dtype == torch.float64) else torch.float32
+    x = input.to(acc).reshape(n1, n2)
+    dout = grad_output.to(acc).reshape(n1, n2)
+    w = weight.to(acc).reshape(1, n2)
+    inv = inv_rms.to(acc).reshape(n1, 1)
+    # cuComputeGradInput, kernel.cu:572-717 (rms_only branch)
+    sum_loss2 = (dout * w * x * inv).sum(-1, keepdim=True)
+    f = n2 * dout * w
+    f = f - x * inv * sum_loss2
+    grad_input = f * ((1.0 / n2) * inv)
+    # cuComputePartGradGammaBeta / cuComputeGradGammaBeta, kernel.cu:402, 444, 520-570
+    grad_weight = (dout * x * inv).sum(0)
+    grad_bias = dout.sum(0) if with_bias else None  # functions_ext.cpp:94-105
+    if exact:
+        return grad_input.reshape(input.shape), grad_weight.reshape(weight.shape), (grad_bias.reshape(weight.shape) if with_bias else None)
+    return (grad_input.to(input.dtype).reshape(input.shape), grad_weight.to(weight.dtype).reshape(weight.shape),
+            grad_bias.to(weight.dtype).reshape(weight.shape) if with_bias else None)
+
+
+def rotary_emb(input: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, conj: bool, interleaved: bool = False, exact: bool = False) -> torch.Tensor:
+    """rotary.cu:26-44: fp32 products (fp64 inputs are narrowed to fp32 too), one rounding to the dtype."""
+    if interleaved:
+        raise NotImplementedError("interleaved rotary embedding is not supported yet")  # functions_ext.cpp:45-48
+    x1, x2 = input.chunk(2, dim=-1)
+    cdt = torch.float64 if exact else torch.float32
+    x1, x2, c, s = x1.to(cdt), x2.to(cdt), cos.to(cdt), sin.to(cdt)
+    if not conj:
+        o1 = x1 * c - x2 * s
+        o2 = x1 * s + x2 * c
+    else:
+        o1 = x1 * c + x2 * s
+        o2 = -x1 * s + x2 * c
+    out = torch.cat((o1, o2), dim=-1)
+    return out if exact else out.to(input.dtype)
+
+
+def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[dest_loc] = k on the raw bytes (numpy), in place; returns out."""
+    nbytes = k.element_size()
+    view_dtype = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[nbytes]
+    o = out.view(view_dtype).numpy()
+    o[dest_loc.numpy().astype(np.int64)] = k.contiguous().view(view_dtype).numpy()
+    return out
+
+
+def _window(b_loc: torch.Tensor, i: int, L: int, max_input_len: int) -> torch.Tensor:
+    """functions_lightllm.cpp:72: the L slots of sequence i are the last L entries of b_loc[i, :max_input_len]."""
+    return b_loc[i].index_select(0, torch.arange(max_input_len - L, max_input_len)).long()
+
+
+def token_attention(q: torch.Tensor, k: torch.Tensor, out: torch.Tensor, b_loc: torch.Tensor, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor,
+                    max_input_len: int, exact: bool = False) -> torch.Tensor:
+    """In place on `out` ([H, cols]); returns it.  With exact=True, `out` must be float64."""
+    batch, head, dim = b_loc.shape[0], q.shape[1], q.shape[2]
+    group = head // k.shape[1]
+    cdt = torch.float64 if exact else q.dtype
+    xq = q.to(cdt).reshape(batch, 1, head, dim).transpose(1, 2)  # [B, H, 1, D]
+    for i in range(batch):
+        L = int(b_seq_len[i])
+        s = int(b_start_loc[i])
+        if L == 0:
+            continue
+        k_loc = _window(b_loc, i, L, max_input_len)
+        key = k[k_loc].to(cdt)  # [L, Hkv, D]
+        if group > 1:
+            key = key.repeat_interleave(group, dim=1)
+        key = key.reshape(1, L, head, dim).transpose(1, 2)  # [1, H, L, D]
+        values = (torch.matmul(xq[i], key.transpose(2, 3)) / math.sqrt(dim)).reshape(head, L)
+        out[:, s:s + L] = values
+    return out
+
+
+def token_softmax_reducev(logics: torch.Tensor, v: torch.Tensor, out: torch.Tensor, b_loc: torch.Tensor, b_start_loc: torch.Tensor,
+                          b_seq_len: torch.Tensor, max_input_len: int, other_kv_index: int = 0, exact: bool = False) -> torch.Tensor:
+    """In place on `out` ([B, H, D]); other_kv_index is ignored like in the reference."""
+    batch, head, dim = b_loc.shape[0], logics.shape[0], v.shape[2]
+    group = head // v.shape[1]
+    cdt = torch.float64 if exact else logics.dtype
+    for i in range(batch):
+        L = int(b_seq_len[i])
+        s = int(b_start_loc[i])
+        if L == 0:
+            continue
+        v_loc = _window(b_loc, i, L, max_input_len)
+        P = logics[:, s:s + L].to(cdt).softmax(-1).reshape(head, 1, 1, L).transpose(0, 1)  # [1, H, 1, L]
+        V = v[v_loc].to(cdt)
+        if group > 1:
+            V = V.repeat_interleave(group, dim=1)
+        V = V.reshape(1, L, head, dim).transpose(1, 2)  # [1, H, L, D]
+        out[i] = torch.matmul(P, V).reshape(head, dim)
+    return out
+
+
+def _torch_context_attention(xq, xk, xv, seqlen, num_head, head_dim, exact):
+    """functions_lightllm.cpp:109-125 with batch size 1."""
+    xq = xq.reshape(1, seqlen, num_head, head_dim).transpose(1, 2)
+    keys = xk.reshape(1, seqlen, num_head, head_dim).transpose(1, 2)
+    values = xv.reshape(1, seqlen, num_head, head_dim).transpose(1, 2)
+    if exact:
+        scores = torch.matmul(xq.double(), keys.double().transpose(2, 3)) / math.sqrt(head_dim)
+        masked = torch.triu(torch.ones(seqlen, seqlen, dtype=torch.bool), diagonal=1)
+        scores = scores.masked_fill(masked, float("-inf")).softmax(-1)
+        return torch.matmul(scores, values.double()).transpose(1, 2).reshape(-1, num_head, head_dim)
+    mask = torch.tril(torch.ones(seqlen, seqlen))
+    mask[mask == 0.0] = -100000000.0  # allowed entries stay +1.0: a constant shift, harmless to softmax
+    scores = torch.matmul(xq, keys.transpose(2, 3)) / math.sqrt(head_dim)
+    scores = torch.softmax(scores.float() + mask, dim=-1).to(xq.dtype)
+    return torch.matmul(scores, values).transpose(1, 2).contiguous().reshape(-1, num_head, head_dim)
+
+
+def context_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor,
+                      max_input_len: int = 0, exact: bool = False) -> torch.Tensor:
+    """In place on `out`; rows outside every sequence are left as they are.  max_input_len is unused (as in the reference)."""
+    batch, head, dim = b_start_loc.shape[0], q.shape[1], q.shape[2]
+    for i in range(batch):
+        start = int(b_start_loc[i])
+        L = int(b_seq_len[i])
+        if L == 0:
+            continue
+        end = start + L
+        out[start:end] = _torch_context_attention(q[start:end], k[start:end], v[start:end], L, head, dim, exact)
+    return out

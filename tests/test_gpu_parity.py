@@ -1,0 +1,488 @@
+"""Parity of the HIP operators (called through the C ABI of libdiopi_impl.so) against the CPU oracle.
+
+Bars (north star): bit-exact for DestIndexCopyKV and all index handling; fp32 within rtol 1e-5
+(atol 1e-5, the reference harness's own default); fp16/bf16 within atol = rtol = 1e-2.  Every case
+also checks that the inputs were not modified, as the reference harness does (case_template.py:205-207).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from diopi_amd import functions as F
+from diopi_amd import runtime as rt
+from diopi_amd import workloads as W
+from oracle import ref_ops as O
+from tests.conftest import TORCH_DTYPES
+from tests.helpers import TOL, assert_bit_equal, assert_close, report
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def snapshot(*tensors):
+    return [None if t is None else t.clone() for t in tensors]
+
+
+def assert_unmodified(before, *tensors):
+    for b, t in zip(before, tensors):
+        if b is not None:
+            assert_bit_equal(t, b, "an input tensor was modified")
+
+
+def test_library_identity():
+    impl = rt.libs().impl
+    assert b"Device" in impl.diopiGetVendorName()
+    assert b"DIOPI Version: 1.0.0" in impl.diopiGetImplVersion()
+    assert rt.device_count() >= 1
+
+
+# ----------------------------------------------------------------------------- DestIndexCopyKV
+def test_destindex_copy_kv_reference_fixtures(golden):
+    g = gen(100)
+    for case in golden["destindex_copy_kv"]["cases"]:
+        for dt in (TORCH_DTYPES[case["dtype"]], torch.bfloat16):
+            for idt in (torch.int32, torch.int64):
+                k = torch.randn(*case["k_shape"], generator=g).to(dt)
+                out = torch.randn(*case["out_shape"], generator=g).to(dt)
+                dest = torch.tensor(case["dest_loc"], dtype=idt)
+                want = O.destindex_copy_kv(k, dest, out.clone())
+                kd, dd, od = k.to(DEV), dest.to(DEV), out.to(DEV)
+                before = snapshot(kd, dd)
+                F.destindex_copy_kv(kd, dd, od)
+                assert_bit_equal(od, want, f"destindex {case['k_shape']} {dt} {idt}")
+                assert_unmodified(before, kd, dd)
+
+
+def test_destindex_copy_kv_config3_shape_bit_exact():
+    w = W.cfg3(DEV, seed=3)
+    for src, cache in ((w["new_k"], w["k_cache"]), (w["new_v"], w["v_cache"])):
+        before_rows = cache[w["dest_loc"].long()].clone()
+        ref = cache.clone()
+        ref[w["dest_loc"].long()] = src  # torch's own scatter on the device as a second opinion
+        sample = torch.randint(0, cache.shape[0], (4096,), generator=gen(1)).to(DEV)
+        untouched_before = cache[sample].clone()
+        F.destindex_copy_kv(src, w["dest_loc"], cache)
+        assert torch.equal(cache.view(torch.int16), ref.view(torch.int16)), "full 1 GiB cache differs from the scatter"
+        # oracle (numpy, CPU) on the touched rows and a sample of untouched ones
+        assert_bit_equal(cache[w["dest_loc"].long()], src, "scattered rows")
+        mask = ~torch.isin(sample, w["dest_loc"].long())
+        assert_bit_equal(cache[sample][mask], untouched_before[mask], "untouched rows")
+        del before_rows
+
+
+def test_destindex_copy_kv_edge_cases():
+    g = gen(101)
+    # odd row sizes exercise every access width; negative indices wrap; out-of-range indices are dropped
+    for shape, dt in (((7, 3, 5), torch.float16), ((6, 1, 3), torch.float32), ((5, 2, 2), torch.float64), ((9, 1, 1), torch.int8), ((4, 33), torch.bfloat16)):
+        k = (torch.randn(*shape, generator=g) * 10).to(dt)
+        rows = 23
+        out = (torch.randn(rows, *shape[1:], generator=g) * 10).to(dt)
+        dest = torch.randperm(rows, generator=g)[: shape[0]].int()
+        want = O.destindex_copy_kv(k, dest, out.clone())
+        od = out.to(DEV)
+        F.destindex_copy_kv(k.to(DEV), dest.to(DEV), od)
+        assert_bit_equal(od, want, f"odd shape {shape} {dt}")
+    k = torch.randn(3, 4, 8, generator=g).half()
+    out = torch.zeros(10, 4, 8).half()
+    od = out.to(DEV)
+    F.destindex_copy_kv(k.to(DEV), torch.tensor([-1, 2, 99], dtype=torch.int32).to(DEV), od)
+    want = out.clone()
+    want[9], want[2] = k[0], k[1]
+    assert_bit_equal(od, want, "negative index wraps, out-of-range index is skipped")
+    # empty token list
+    F.destindex_copy_kv(torch.zeros(0, 4, 8, dtype=torch.float16, device=DEV), torch.zeros(0, dtype=torch.int32, device=DEV), od)
+    assert_bit_equal(od, want, "empty scatter")
+
+
+def test_destindex_copy_kv_large_round_trip():
+    # encode -> scatter -> gather round trip over a full permutation of 65536 rows of 8 KiB
+    T = 65536
+    src = torch.randint(-32768, 32767, (T, 32, 128), dtype=torch.int16, device=DEV).view(torch.float16)
+    perm = torch.randperm(T, device=DEV).int()
+    cache = torch.zeros_like(src)
+    F.destindex_copy_kv(src, perm, cache)
+    assert torch.equal(cache[perm.long()].view(torch.int16), src.view(torch.int16))
+
+
+# ----------------------------------------------------------------------------- RMSNorm
+def _rms_case(shape, ns, eps, dt, with_bias, seed, ones_grad):
+    g = gen(seed)
+    x = torch.randn(*shape, generator=g).to(dt)
+    w = (torch.rand(*ns, generator=g) + 0.5).to(dt)
+    b = torch.randn(*ns, generator=g).to(dt) if with_bias else None
+    go = torch.ones(*shape).to(dt) if ones_grad else torch.randn(*shape, generator=g).to(dt)
+    xd, wd, bd, god = x.to(DEV), w.to(DEV), (b.to(DEV) if with_bias else None), go.to(DEV)
+    before = snapshot(xd, wd, bd, god)
+    out = F.rms_norm(xd, ns, wd, bd, eps)
+    inv = F.GLOBAL_STATE["rms_norm_inv_rms"]
+    grads = F.rms_norm_backward([god], xd, wd, bd, ns, eps)
+    assert_unmodified(before, xd, wd, bd, god)
+    ref_out, ref_inv = O.rms_norm(x, ns, w, b, eps)
+    ex_out, ex_inv = O.rms_norm(x, ns, w, b, eps, exact=True)
+    tol = TOL[dt]
+    what = f"rms_norm {shape} ns={ns} {dt} bias={with_bias}"
+    assert inv.dtype == (torch.float64 if dt == torch.float64 else torch.float32) and tuple(inv.shape) == tuple(ref_inv.shape)
+    assert_close(inv, ex_inv, 1e-6 if dt != torch.float64 else 1e-12, 0, what + " inv_rms")
+    assert_close(out, ref_out, what=what + " out vs reference composition", **tol)
+    if with_bias and dt in (torch.float16, torch.bfloat16):
+        # the reference rounds weight*normed to 16 bits before adding the bias: where the sum cancels, the distance to the
+        # float64 value is one rounding of the larger intermediate, not of the result
+        mag = float((ex_out - b.double()).abs().max())
+        assert_close(out, ex_out, rtol=tol["rtol"], atol=max(tol["atol"], mag * 2.0 ** -8), what=what + " out vs float64")
+    else:
+        assert_close(out, ex_out, what=what + " out vs float64", **tol)
+    # backward is checked with the inv_rms the device produced, as the harness feeds it back
+    r_gi, r_gw, r_gb = O.rms_norm_backward(go, x, w, inv.cpu(), ns, with_bias=with_bias)
+    e_gi, e_gw, e_gb = O.rms_norm_backward(go, x, w, inv.cpu(), ns, with_bias=with_bias, exact=True)
+    n1 = x.numel() // int(np.prod(ns))
+    assert_close(grads["input"], r_gi, what=what + " grad_input", **tol)
+    assert_close(grads["input"], e_gi, what=what + " grad_input vs float64", **tol)
+    # a column sum over n1 rows: the reference's own fp32 summation order moves the result by ~1e-7*sqrt(n1)*|terms|,
+    # so the fp32 comparison against the float64 sum carries an absolute term scaled by the size of the sum
+    scale = float((go.double() * x.double()).abs().sum(tuple(range(x.dim() - len(ns)))).max()) if n1 > 0 else 1.0
+    atol_w = tol["atol"] if dt != torch.float32 else max(1e-5, 2e-7 * scale)
+    assert_close(grads["weight"], e_gw, rtol=tol["rtol"], atol=atol_w, what=what + " grad_weight vs float64")
+    if dt in (torch.float16, torch.bfloat16):
+        # 16-bit outputs of sums over many rows: one rounding of the exact sum
+        assert_close(grads["weight"], r_gw, rtol=1e-2, atol=max(1e-2, 8e-3 * float(e_gw.abs().max())), what=what + " grad_weight vs reference")
+    if with_bias:
+        assert_close(grads["bias"], e_gb, rtol=tol["rtol"], atol=max(atol_w, tol["atol"]), what=what + " grad_bias")
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_rms_norm_reference_cases(golden, dtype):
+    dt = TORCH_DTYPES[dtype]
+    for i, case in enumerate(golden["rms_norm"]["cases"]):
+        for with_bias in (False, True):
+            say("rms_norm case", case, dtype, with_bias)
+            _rms_case(tuple(case["input"]), tuple(case["normalized_shape"]), case["eps"], dt, with_bias, 200 + i, ones_grad=(i % 2 == 0))
+
+
+@pytest.mark.parametrize("shape,dtype", [((512, 4096), "float32"), ((300, 4096), "bfloat16"), ((129, 8192), "float16"), ((64, 1024), "float32"),
+                                         ((33, 2048), "float16"), ((17, 4104), "float32"), ((8, 16384), "float32"), ((5, 40000), "float16")])
+def test_rms_norm_wide_rows(shape, dtype):
+    say("rms_norm wide", shape, dtype)
+    _rms_case(shape, (shape[-1],), 1e-6, TORCH_DTYPES[dtype], with_bias=(shape[0] % 2 == 1), seed=300, ones_grad=False)
+
+
+def test_rms_norm_config1_full_size():
+    w = W.cfg1(DEV, seed=1)
+    x, wt, go = w["x"], w["weight"], w["grad_out"]
+    out = F.rms_norm(x, w["normalized_shape"], wt, None, w["eps"])
+    inv = F.GLOBAL_STATE["rms_norm_inv_rms"]
+    grads = F.rms_norm_backward([go], x, wt, None, w["normalized_shape"], w["eps"])
+    xc, wc, goc = x.cpu(), wt.cpu(), go.cpu()
+    ref_out, ref_inv = O.rms_norm(xc, w["normalized_shape"], wc, None, w["eps"])
+    assert_close(out, ref_out, rtol=1e-5, atol=1e-5, what="cfg1 out")
+    assert_close(inv, ref_inv, rtol=1e-5, atol=0, what="cfg1 inv_rms")
+    e_gi, e_gw, _ = O.rms_norm_backward(goc, xc, wc, inv.cpu(), w["normalized_shape"], exact=True)
+    r_gi, r_gw, _ = O.rms_norm_backward(goc, xc, wc, inv.cpu(), w["normalized_shape"])
+    assert_close(grads["input"], r_gi, rtol=1e-5, atol=1e-5, what="cfg1 grad_input")
+    # grad_weight: against the float64 column sum at rtol 1e-5 with an absolute floor of one part in 1e7 of sum|terms|
+    floor = 2e-7 * float((goc.double() * xc.double() * inv.cpu().double()[:, None]).abs().sum(0).max())
+    assert_close(grads["weight"], e_gw, rtol=1e-5, atol=floor, what="cfg1 grad_weight vs float64")
+    say("cfg1 grad_weight: max_abs/max_rel vs float64 %.3e %.3e ; reference fp32 order vs float64 %.3e %.3e" %
+        (report(grads["weight"], e_gw) + report(r_gw, e_gw)))
+    # the reference harness's own bar for rms_norm (atol = rtol = 1e-4) against the fp32 ATen result
+    assert_close(grads["weight"], r_gw, rtol=1e-4, atol=1e-4, what="cfg1 grad_weight vs fp32 ATen")
+
+
+def test_rms_norm_config2_full_size():
+    w = W.cfg2(DEV, seed=2)
+    out = F.rms_norm(w["x"], w["normalized_shape"], w["weight"], None, w["eps"])
+    ref_out, ref_inv = O.rms_norm(w["x"].cpu(), w["normalized_shape"], w["weight"].cpu(), None, w["eps"])
+    assert_close(out, ref_out, rtol=1e-2, atol=1e-2, what="cfg2 rms_norm bf16")
+    assert_close(F.GLOBAL_STATE["rms_norm_inv_rms"], ref_inv, rtol=1e-5, atol=0, what="cfg2 inv_rms")
+    # mixed precision pair of the reference: fp32 input, 16-bit output and weight
+    x32 = w["x"][:257].float()
+    o16 = F.rms_norm(x32, w["normalized_shape"], w["weight"], None, w["eps"], out_dtype=torch.bfloat16)
+    r16, _ = O.rms_norm(x32.cpu(), w["normalized_shape"], w["weight"].cpu(), None, w["eps"], out_dtype=torch.bfloat16)
+    assert_close(o16, r16, rtol=1e-2, atol=1e-2, what="fp32 -> bf16 rms_norm")
+
+
+# ----------------------------------------------------------------------------- Rotary
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_rotary_reference_cases(golden, dtype):
+    dt = TORCH_DTYPES[dtype]
+    g = gen(400)
+    for case in golden["rotary_emb"]["cases"] + golden["rotary_emb"]["empty_cases"]:
+        say("rotary case", case, dtype)
+        x = torch.randn(*case["input"], generator=g).to(dt)
+        cos = torch.randn(*case["cos"], generator=g).to(dt)
+        sin = torch.randn(*case["cos"], generator=g).to(dt)
+        xd, cd, sd = x.to(DEV), cos.to(DEV), sin.to(DEV)
+        before = snapshot(xd, cd, sd)
+        if case["interleaved"]:
+            with pytest.raises(rt.FunctionNotImplementedError):  # the harness turns code 13 into a skip
+                F.rotary_emb(xd, cd, sd, case["conj"], True)
+            continue
+        out = F.rotary_emb(xd, cd, sd, case["conj"], False)
+        assert_unmodified(before, xd, cd, sd)
+        ref = O.rotary_emb(x, cos, sin, case["conj"])
+        if dt == torch.float64:
+            assert_close(out, ref, rtol=1e-6, atol=1e-6, what=f"rotary {case}")  # fp32 products, as the reference computes them
+        else:
+            assert_close(out, ref, what=f"rotary {case}", **TOL[dt])
+
+
+def test_rotary_position_zero_identity_and_inverse():
+    g = gen(401)
+    x = torch.randn(64, 32, 128, generator=g).half().to(DEV)
+    one = torch.ones(64, 1, 64, dtype=torch.float16, device=DEV)
+    zero = torch.zeros_like(one)
+    assert_bit_equal(F.rotary_emb(x, one, zero, False, False), x, "angle 0 is the identity")
+    ang = torch.rand(64, 1, 64, generator=g) * 6.28
+    xf = x.float()
+    y = F.rotary_emb(xf, ang.cos().to(DEV), ang.sin().to(DEV), False, False)
+    back = F.rotary_emb(y, ang.cos().to(DEV), ang.sin().to(DEV), True, False)
+    assert_close(back, xf, rtol=1e-5, atol=1e-5, what="conj inverts the rotation")
+
+
+def test_rotary_config2_full_size():
+    w = W.cfg2(DEV, seed=2)
+    for name in ("q", "k"):
+        out = F.rotary_emb(w[name], w["cos"], w["sin"], False, False)
+        ref = O.rotary_emb(w[name].cpu(), w["cos"].cpu(), w["sin"].cpu(), False)
+        # one rounding of an fp32 result on both sides: the results agree to the last bit almost everywhere
+        assert_close(out, ref, rtol=1e-2, atol=1e-2, what=f"cfg2 rotary {name}")
+        same = float((out.cpu().view(torch.int16) == ref.view(torch.int16)).float().mean())
+        say(f"cfg2 rotary {name}: bit-identical fraction {same:.6f}")
+        assert same > 0.999
+
+
+# ----------------------------------------------------------------------------- decode attention
+def _decode_case(w, dtype, what, seq_subset=None):
+    """token_attention then token_softmax_reducev on workload dict `w`; oracle on the CPU for `seq_subset` sequences."""
+    q, kc, vc = w["q"], w["k_cache"], w["v_cache"]
+    H, total = q.shape[1], w["total_len"]
+    tol = TOL[dtype]
+    logits = torch.full((H, total), -12288.0, dtype=dtype, device=DEV)
+    before = snapshot(q, w["b_loc"], w["b_start_loc"], w["b_seq_len"])
+    F.token_attention(q, kc, logits, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
+    out = torch.zeros_like(q)
+    F.token_softmax_reducev(logits, vc, out, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], 0)
+    assert_unmodified(before, q, w["b_loc"], w["b_start_loc"], w["b_seq_len"])
+    idx = list(range(q.shape[0])) if seq_subset is None else seq_subset
+    sel = torch.tensor(idx)
+    # the oracle gathers only the cache rows it needs: remap slots of the chosen sequences to a compact cache
+    b_loc_c, b_len_c, b_start_c = w["b_loc"].cpu()[sel], w["b_seq_len"].cpu()[sel], w["b_start_loc"].cpu()[sel]
+    used = torch.unique(b_loc_c.long())
+    remap = torch.zeros(int(used.max()) + 1, dtype=torch.int32)
+    remap[used] = torch.arange(used.numel(), dtype=torch.int32)
+    loc_small = remap[b_loc_c.long()]
+    k_small, v_small = kc[used.to(DEV)].cpu(), vc[used.to(DEV)].cpu()
+    ref_logits = torch.full((H, total), -12288.0, dtype=dtype)
+    O.token_attention(q.cpu()[sel], k_small, ref_logits, loc_small, b_start_c, b_len_c, w["max_input_len"])
+    ex_logits = torch.full((H, total), -12288.0, dtype=torch.float64)
+    O.token_attention(q.cpu()[sel], k_small, ex_logits, loc_small, b_start_c, b_len_c, w["max_input_len"], exact=True)
+    cols = torch.cat([torch.arange(int(s), int(s) + int(L)) for s, L in zip(b_start_c, b_len_c)])
+    dev_logits = logits.cpu()
+    assert_close(dev_logits[:, cols], ref_logits[:, cols], what=what + " logits vs reference composition", **tol)
+    assert_close(dev_logits[:, cols], ex_logits[:, cols], what=what + " logits vs float64", **tol)
+    if seq_subset is None:
+        assert_bit_equal(dev_logits, torch.where(ref_logits == -12288.0, ref_logits, dev_logits), what + ": columns outside every sequence were written")
+    # second operator: feed the oracle the device's logits so that the two checks are independent
+    ref_out = torch.zeros(len(idx), H, q.shape[2], dtype=dtype)
+    O.token_softmax_reducev(dev_logits, v_small, ref_out, loc_small, b_start_c, b_len_c, w["max_input_len"], 0)
+    ex_out = torch.zeros(len(idx), H, q.shape[2], dtype=torch.float64)
+    O.token_softmax_reducev(dev_logits, v_small, ex_out, loc_small, b_start_c, b_len_c, w["max_input_len"], 0, exact=True)
+    assert_close(out.cpu()[sel], ref_out, what=what + " out vs reference composition", **tol)
+    assert_close(out.cpu()[sel], ex_out, what=what + " out vs float64", **tol)
+    say(what, "logits max_abs/rel vs f64: %.3e %.3e" % report(dev_logits[:, cols], ex_logits[:, cols]), " out: %.3e %.3e" % report(out.cpu()[sel], ex_out))
+    return logits, out
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "bfloat16", "float64"])
+def test_decode_reference_fixture(golden, dtype):
+    dt = TORCH_DTYPES[dtype]
+    fx = golden["token_attention"]
+    g = gen(500)
+    w = dict(q=torch.randn(*fx["q_shape"], generator=g).to(dt).to(DEV), k_cache=torch.randn(*fx["k_shape"], generator=g).to(dt).to(DEV),
+             v_cache=torch.randn(*fx["k_shape"], generator=g).to(dt).to(DEV), b_loc=torch.tensor(fx["b_loc"], dtype=torch.int32, device=DEV),
+             b_start_loc=torch.tensor(fx["b_start_loc"], dtype=torch.int32, device=DEV), b_seq_len=torch.tensor(fx["b_seq_len"], dtype=torch.int32, device=DEV),
+             max_input_len=fx["max_input_len"], total_len=13)
+    _decode_case(w, dt, f"decode fixture {dtype}")
+
+
+def test_decode_index_exactness_and_int64():
+    # k[slot] = slot pattern: the logits are exact small integers times a constant, so any wrong slot shows up exactly
+    D, H = 128, 32
+    slots = 300
+    k = (torch.arange(slots, dtype=torch.float32) % 61).reshape(slots, 1, 1).expand(slots, H, D).contiguous().half().to(DEV)
+    k = k * (torch.arange(D, device=DEV) == 0)  # only dim 0 is non-zero -> q.k = slot % 61 exactly
+    q = torch.ones(3, H, D, dtype=torch.float16, device=DEV)
+    rng = np.random.Generator(np.random.PCG64(7))
+    b_len = np.array([1, 130, 77])
+    b_start = np.array([0, 1, 131])
+    b_loc = rng.permutation(slots)[: 3 * 90].reshape(3, 90)
+    b_loc = np.concatenate([b_loc, rng.permutation(slots)[: 3 * 60].reshape(3, 60)], axis=1)  # width 150
+    for idt in (torch.int32, torch.int64):
+        out = torch.zeros(H, 208, dtype=torch.float16, device=DEV)
+        F.token_attention(q, k, out, torch.from_numpy(b_loc).to(idt).to(DEV), torch.from_numpy(b_start).to(idt).to(DEV),
+                          torch.from_numpy(b_len).to(idt).to(DEV), 140)
+        want = np.concatenate([b_loc[i, 140 - L:140] % 61 for i, L in enumerate(b_len)]).astype(np.float32)
+        want = torch.tensor(want).half().float() * (1.0 / math.sqrt(D))
+        # a wrong slot moves a logit by at least 1/sqrt(128) = 0.088
+        assert_close(out.cpu(), want.half().expand(H, 208), rtol=0, atol=1e-3, what=f"slot pattern {idt}")
+
+
+def test_decode_config3_scaled_and_ragged():
+    w = W.cfg3(DEV, seed=3, scale=0.125)  # 8 sequences of 512..2048 tokens
+    _decode_case(w, torch.float16, "cfg3 x 1/8")
+    # ragged: lengths 1, 15, 16, 17, 127, 128, 129, 257 and one empty sequence
+    lens = np.array([1, 15, 16, 17, 0, 127, 128, 129, 257], dtype=np.int32)
+    B = len(lens)
+    w2 = W._decode(DEV, 33, torch.float16, B, 32, 32, 128, 4096, 1, 300, B)
+    w2["b_seq_len"] = torch.from_numpy(lens).to(DEV)
+    w2["b_start_loc"] = torch.from_numpy(np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int32)).to(DEV)
+    w2["total_len"] = int(lens.sum())
+    w2["max_input_len"] = 260
+    _decode_case(w2, torch.float16, "ragged lengths")
+
+
+def test_decode_gqa_config5_scaled():
+    w = W.cfg5(DEV, seed=5, scale=1 / 32)  # 4 sequences of 1024..8192 tokens, 64 q heads over 8 kv heads
+    _decode_case(w, torch.bfloat16, "cfg5 x 1/32")
+    for G, Hkv in ((2, 4), (4, 2), (16, 1), (3, 2)):
+        w3 = W._decode(DEV, 55 + G, torch.float16, 3, G * Hkv, Hkv, 128, 2048, 5, 600, 3)
+        _decode_case(w3, torch.float16, f"GQA G={G} Hkv={Hkv}")
+
+
+def test_decode_config3_full_size_sampled():
+    w = W.cfg3(DEV, seed=3)
+    logits, out = _decode_case(w, torch.float16, "cfg3 full, 6 sequences checked", seq_subset=[0, 7, 21, 40, 62, 63])
+    # size-independent properties over the whole batch: constant logits give the mean of the gathered rows,
+    # and the result is invariant under a relabelling of the cache slots
+    const = torch.zeros_like(logits)
+    o2 = torch.zeros_like(out)
+    F.token_softmax_reducev(const, w["v_cache"], o2, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], 0)
+    i = 17
+    L = int(w["b_seq_len"][i])
+    rows = w["b_loc"][i, w["max_input_len"] - L: w["max_input_len"]].long()
+    assert_close(o2[i], w["v_cache"][rows].float().mean(0), rtol=1e-2, atol=1e-2, what="uniform softmax = mean of rows")
+    perm = torch.randperm(w["slots"], device=DEV)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(w["slots"], device=DEV)
+    k2 = torch.empty_like(w["k_cache"])
+    k2[perm] = w["k_cache"]
+    l2 = torch.zeros_like(logits)
+    F.token_attention(w["q"], k2, l2, perm[w["b_loc"].long()].int(), w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
+    assert_bit_equal(l2, logits, "relabelling the cache slots changes nothing")
+
+
+def test_decode_config5_full_size_sampled():
+    w = W.cfg5(DEV, seed=5)
+    _decode_case(w, torch.bfloat16, "cfg5 full, 3 sequences checked", seq_subset=[0, 64, 127])
+
+
+# ----------------------------------------------------------------------------- prefill attention
+def _context_case(q, k, v, b_start, b_len, max_len, dt, what, check_rows=None):
+    T = q.shape[0]
+    out = torch.full_like(q, 77.0)
+    before = snapshot(q, k, v, b_start, b_len)
+    F.context_attention(q, k, v, out, b_start, b_len, max_len)
+    assert_unmodified(before, q, k, v, b_start, b_len)
+    tol = TOL[dt]
+    outc = out.cpu()
+    covered = torch.zeros(T, dtype=torch.bool)
+    for s, L in zip(b_start.tolist(), b_len.tolist()):
+        covered[s:s + L] = True
+        if L > 0:
+            assert_bit_equal(outc[s], v[s].cpu(), what + ": the first token of a sequence returns its own v row")
+    assert bool((outc[~covered] == 77.0).all()), what + ": rows outside every sequence were written"
+    if check_rows is None:
+        ref = torch.full(q.shape, 77.0, dtype=dt)
+        O.context_attention(q.cpu(), k.cpu(), v.cpu(), ref, b_start.cpu(), b_len.cpu(), max_len)
+        ex = torch.full(q.shape, 77.0, dtype=torch.float64)
+        O.context_attention(q.cpu(), k.cpu(), v.cpu(), ex, b_start.cpu(), b_len.cpu(), max_len, exact=True)
+        # the reference narrows the scores to fp32 for its softmax whatever the tensor dtype (functions_lightllm.cpp:122),
+        # so for float64 tensors its own result is only fp32-accurate
+        rtol_ref = dict(rtol=1e-6, atol=1e-6) if dt == torch.float64 else tol
+        assert_close(outc, ref, what=what + " vs reference composition", **rtol_ref)
+        assert_close(outc, ex, what=what + " vs float64", **tol)
+        say(what, "max_abs/rel vs f64: %.3e %.3e" % report(outc, ex))
+    else:
+        # full-size inputs: float64 attention for sampled rows only (decode formulation of the same row)
+        kc, vc = k.cpu(), v.cpu()
+        for (i, r) in check_rows:
+            s = int(b_start[i])
+            qq = q[s + r: s + r + 1].cpu()
+            loc = torch.arange(s, s + r + 1, dtype=torch.int32).reshape(1, -1)
+            lg = torch.zeros(q.shape[1], r + 1, dtype=torch.float64)
+            O.token_attention(qq, kc, lg, loc, torch.tensor([0]), torch.tensor([r + 1]), r + 1, exact=True)
+            ex = torch.zeros(1, q.shape[1], q.shape[2], dtype=torch.float64)
+            O.token_softmax_reducev(lg, vc, ex, loc, torch.tensor([0]), torch.tensor([r + 1]), r + 1, 0, exact=True)
+            assert_close(outc[s + r], ex[0], what=f"{what} sequence {i} row {r} vs float64", **tol)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_context_attention_reference_fixtures(golden, dtype):
+    dt = TORCH_DTYPES[dtype]
+    g = gen(600)
+    for case in golden["context_attention"]["cases"]:
+        say("context case", case, dtype)
+        q, k, v = ((torch.randn(*case["shape"], generator=g) * 0.5).to(dt).to(DEV) for _ in range(3))
+        bs = torch.tensor(case["b_start_loc"], dtype=torch.int32, device=DEV)
+        bl = torch.tensor(case["b_seq_len"], dtype=torch.int32, device=DEV)
+        _context_case(q, k, v, bs, bl, case["max_input_len"], dt, f"context {case['shape']} {dtype}")
+
+
+def test_context_attention_ragged_lengths():
+    g = gen(601)
+    lens = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 193, 300]
+    starts, pos = [], 3  # a gap before the first sequence and between some of them
+    for i, L in enumerate(lens):
+        starts.append(pos)
+        pos += L + (5 if i % 3 == 0 else 0)
+    T = pos + 4
+    for dt in (torch.float16, torch.bfloat16):
+        q, k, v = ((torch.randn(T, 4, 128, generator=g) * 0.5).to(dt).to(DEV) for _ in range(3))
+        for idt in (torch.int32, torch.int64):
+            _context_case(q, k, v, torch.tensor(starts, dtype=idt, device=DEV), torch.tensor(lens, dtype=idt, device=DEV), max(lens), dt,
+                          f"ragged {dt} {idt}")
+
+
+def test_context_attention_config4_scaled():
+    w = W.cfg4(DEV, seed=4, scale=0.125)  # 8 sequences of 128..512 tokens
+    _context_case(w["q"], w["k"], w["v"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], torch.float16, "cfg4 x 1/8")
+
+
+def test_context_attention_config4_full_size_sampled():
+    w = W.cfg4(DEV, seed=4)
+    rows = []
+    rng = np.random.Generator(np.random.PCG64(9))
+    for i, L in enumerate(w["seq_len_host"].tolist()):
+        rows += [(i, L - 1), (i, int(rng.integers(0, L))), (i, min(L - 1, 127)), (i, min(L - 1, 128))]
+    out = _context_case(w["q"], w["k"], w["v"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], torch.float16, "cfg4 full", check_rows=rows)
+    # constant V per head => the output equals V whatever the scores are
+    vconst = w["v"][:1].expand_as(w["v"]).contiguous()
+    o2 = torch.zeros_like(out)
+    F.context_attention(w["q"], w["k"], vconst, o2, w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
+    assert_close(o2, vconst, rtol=1e-2, atol=1e-3, what="cfg4 full, constant V")
+
+
+# ----------------------------------------------------------------------------- error behaviour on a GPU box
+def test_errors_do_not_launch():
+    x = torch.randn(4, 8, device=DEV)
+    w = torch.ones(8, device=DEV)
+    before = rt.get_last_error_string()
+    with pytest.raises(rt.DiopiException):
+        F.rms_norm(x, (7,), w, None, 1e-6)  # normalized_shape does not match
+    assert rt.get_last_error_string() != before
+    with pytest.raises(rt.DiopiException):
+        F.rms_norm(x.t(), (4,), torch.ones(4, device=DEV), None, 1e-6)  # non-contiguous input is rejected, not converted
+    with pytest.raises(rt.DiopiException):
+        F.destindex_copy_kv(x.half(), torch.zeros(4, dtype=torch.int32, device=DEV), x)  # dtype mismatch
+    torch.cuda.synchronize()

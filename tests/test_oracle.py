@@ -1,0 +1,361 @@
+"""Pins the CPU oracle (oracle/ref_ops.py) against what the reference's own fixtures and the
+mathematics fix, so that a dropped term, a wrong sign/index or a transposed operand fails here.
+Runs on the CPU; no GPU, no product code."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ref_ops as O
+from tests.conftest import TORCH_DTYPES
+from tests.helpers import assert_bit_equal, assert_close
+
+
+def rng(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ----------------------------------------------------------------------------- rms_norm
+def test_rms_norm_constant_rows_closed_form():
+    # x == c  =>  inv_rms = 1/sqrt(c^2 + eps), out = w * c * inv_rms
+    c, eps = 3.0, 1e-2
+    x = torch.full((7, 16), c, dtype=torch.float64)
+    w = torch.linspace(0.5, 1.5, 16, dtype=torch.float64)
+    out, inv = O.rms_norm(x, (16,), w, None, eps)
+    assert_close(inv, torch.full((7,), 1 / math.sqrt(c * c + eps), dtype=torch.float64), 1e-14, 0, "inv_rms")
+    assert_close(out, (w * c / math.sqrt(c * c + eps)).expand(7, 16), 1e-14, 0, "out")
+
+
+def test_rms_norm_sign_rows_and_scale_invariance():
+    g = rng(0)
+    x = (torch.randint(0, 2, (5, 32), generator=g) * 2 - 1).double()
+    out, inv = O.rms_norm(x, (32,), torch.ones(32, dtype=torch.float64), None, 1e-6)
+    assert_close(out, x / math.sqrt(1 + 1e-6), 1e-14, 0, "+-1 rows")
+    # eps = 0: out(a*x) == out(x)
+    y = torch.randn(4, 24, generator=g, dtype=torch.float64)
+    w = torch.rand(24, generator=g, dtype=torch.float64) + 0.5
+    o1, _ = O.rms_norm(y, (24,), w, None, 0.0)
+    o2, _ = O.rms_norm(y * 7.5, (24,), w, None, 0.0)
+    assert_close(o1, o2, 1e-13, 0, "scale invariance")
+
+
+def test_rms_norm_energy_identity_and_bias_and_multidim():
+    g = rng(1)
+    x = torch.randn(3, 2, 7, 8, generator=g, dtype=torch.float64)
+    w = torch.rand(7, 8, generator=g, dtype=torch.float64) + 0.5
+    b = torch.randn(7, 8, generator=g, dtype=torch.float64)
+    eps = 1e-2
+    out, inv = O.rms_norm(x, (7, 8), w, None, eps)
+    ms = (x * x).mean(dim=(-1, -2))
+    # sum((out/w)^2) = n2 * ms / (ms + eps)
+    assert_close(((out / w) ** 2).sum(dim=(-1, -2)), 56 * ms / (ms + eps), 1e-12, 0, "energy identity")
+    assert tuple(inv.shape) == (3, 2)
+    out_b, _ = O.rms_norm(x, (7, 8), w, b, eps)
+    assert_close(out_b - out, b.expand_as(out), 1e-12, 1e-14, "bias is added after the scaling")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_rms_norm_modes_agree_and_match_python_twin(dtype):
+    # the reference's Python statement (customized_test.py:392-403): weight * (x * rsqrt(mean(x^2) + eps))
+    g = rng(2)
+    x = torch.randn(35, 125, 32, generator=g).to(dtype)
+    w = (torch.rand(32, generator=g) + 0.5).to(dtype)
+    out, inv = O.rms_norm(x, (32,), w, None, 1e-6)
+    twin = (w.float() * (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6))).to(dtype)
+    exact, inv64 = O.rms_norm(x, (32,), w, None, 1e-6, exact=True)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    assert_close(out, twin, tol, tol, "kernel statement vs python statement")
+    assert_close(out, exact, tol, tol, "dtype-faithful vs float64")
+    assert inv.dtype == torch.float32 and out.dtype == dtype
+
+
+def test_rms_norm_backward_matches_float64_autograd():
+    g = rng(3)
+    for shape, ns in [((5, 5), (5,)), ((16, 64, 64), (64, 64)), ((3, 2, 16, 7, 8), (7, 8))]:
+        x = torch.randn(*shape, generator=g, dtype=torch.float64, requires_grad=True)
+        w = (torch.rand(*ns, generator=g, dtype=torch.float64) + 0.5).requires_grad_()
+        b = torch.randn(*ns, generator=g, dtype=torch.float64, requires_grad=True)
+        go = torch.randn(*shape, generator=g, dtype=torch.float64)
+        eps = 1e-4
+        dims = tuple(range(-len(ns), 0))
+        y = w * (x * torch.rsqrt((x * x).mean(dims, keepdim=True) + eps)) + b  # textbook RMSNorm
+        gx, gw, gb = torch.autograd.grad(y, (x, w, b), go)
+        _, inv = O.rms_norm(x.detach(), ns, w.detach(), None, eps)
+        ox, ow, ob = O.rms_norm_backward(go, x.detach(), w.detach(), inv, ns, with_bias=True)
+        assert_close(ox, gx, 1e-10, 1e-12, "grad_input")
+        assert_close(ow, gw, 1e-10, 1e-12, "grad_weight")
+        assert_close(ob, gb, 1e-10, 1e-12, "grad_bias")
+
+
+def test_rms_norm_backward_orthogonality_identity():
+    # sum_l x_l * grad_input_l = eps * inv_rms^3 * sum_l g_l x_l   (zero for eps = 0)
+    g = rng(4)
+    x = torch.randn(9, 40, generator=g, dtype=torch.float64)
+    w = torch.rand(40, generator=g, dtype=torch.float64) + 0.5
+    go = torch.randn(9, 40, generator=g, dtype=torch.float64)
+    for eps in (0.0, 1e-2):
+        _, inv = O.rms_norm(x, (40,), w, None, eps)
+        gx, _, _ = O.rms_norm_backward(go, x, w, inv, (40,))
+        lhs = (x * gx).sum(-1)
+        rhs = eps * inv ** 3 * (go * w * x).sum(-1)
+        assert_close(lhs, rhs, 1e-9, 1e-12, f"identity eps={eps}")
+
+
+# ----------------------------------------------------------------------------- rotary
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32, torch.float64])
+def test_rotary_position_zero_is_identity_bitwise(dtype):
+    g = rng(5)
+    x = torch.randn(1, 9, 4, 32, generator=g).to(dtype)
+    cos = torch.ones(9, 1, 16, dtype=dtype)
+    sin = torch.zeros(9, 1, 16, dtype=dtype)
+    for conj in (False, True):
+        assert_bit_equal(O.rotary_emb(x, cos, sin, conj), x, "rotation by angle 0")
+
+
+def test_rotary_norm_preserved_and_conj_inverts_and_quarter_turn():
+    g = rng(6)
+    x = torch.randn(3, 100, 8, 64, generator=g, dtype=torch.float64)
+    ang = torch.rand(100, 1, 32, generator=g, dtype=torch.float64) * 6.28
+    cos, sin = ang.cos(), ang.sin()
+    y = O.rotary_emb(x, cos, sin, False, exact=True)
+    x1, x2 = x.chunk(2, -1)
+    y1, y2 = y.chunk(2, -1)
+    assert_close(y1 ** 2 + y2 ** 2, x1 ** 2 + x2 ** 2, 1e-12, 1e-14, "pairwise norm")
+    assert_close(O.rotary_emb(y, cos, sin, True, exact=True), x, 1e-12, 1e-14, "conj undoes the rotation")
+    # a quarter turn (c=0, s=1) maps (x1, x2) -> (-x2, x1); with conj -> (x2, -x1): pins signs and operand order
+    q = O.rotary_emb(x, torch.zeros_like(cos), torch.ones_like(sin), False, exact=True)
+    assert_close(q, torch.cat((-x2, x1), -1), 0, 0, "quarter turn")
+    qc = O.rotary_emb(x, torch.zeros_like(cos), torch.ones_like(sin), True, exact=True)
+    assert_close(qc, torch.cat((x2, -x1), -1), 0, 0, "quarter turn, conj")
+
+
+def test_rotary_reference_shapes_broadcast(golden):
+    g = rng(7)
+    for case in golden["rotary_emb"]["cases"] + golden["rotary_emb"]["empty_cases"]:
+        x = torch.randn(*case["input"], generator=g)
+        cos = torch.randn(*case["cos"], generator=g)
+        sin = torch.randn(*case["cos"], generator=g)
+        if case["interleaved"]:
+            with pytest.raises(NotImplementedError):
+                O.rotary_emb(x, cos, sin, case["conj"], True)
+            continue
+        out = O.rotary_emb(x, cos, sin, case["conj"])
+        assert out.shape == x.shape
+        if x.numel():
+            # spot check one element with explicit index arithmetic (right-aligned broadcast)
+            half = x.shape[-1] // 2
+            idx = tuple(s - 1 for s in x.shape[:-1])
+            cidx = tuple(min(i, s - 1) for i, s in zip(idx[len(idx) - (cos.dim() - 1):], cos.shape[:-1])) if cos.dim() > 1 else ()
+            c, s_ = float(cos[cidx + (0,)]), float(sin[cidx + (0,)])
+            a, b = float(x[idx + (0,)]), float(x[idx + (half,)])
+            want = a * c + b * s_ if case["conj"] else a * c - b * s_
+            assert abs(float(out[idx + (0,)]) - want) < 1e-5
+
+
+def test_rotary_fp64_is_computed_in_fp32():
+    # rotary.cu:30-43 narrows every operand with static_cast<float>, also for double tensors
+    x = torch.tensor([1.0 + 2 ** -40, 3.0], dtype=torch.float64)
+    out = O.rotary_emb(x, torch.ones(1, dtype=torch.float64), torch.zeros(1, dtype=torch.float64), False)
+    assert float(out[0]) == 1.0
+
+
+# ----------------------------------------------------------------------------- destindex_copy_kv
+def test_destindex_copy_kv_reference_fixtures(golden):
+    g = rng(8)
+    for case in golden["destindex_copy_kv"]["cases"]:
+        dt = TORCH_DTYPES[case["dtype"]]
+        k = torch.randn(*case["k_shape"], generator=g).to(dt)
+        out = torch.randn(*case["out_shape"], generator=g).to(dt)
+        before = out.clone()
+        dest = torch.tensor(case["dest_loc"], dtype=torch.int32)
+        O.destindex_copy_kv(k, dest, out)
+        touched = set(case["dest_loc"])
+        for t, d in enumerate(case["dest_loc"]):
+            assert_bit_equal(out[d], k[t], f"row {d}")
+        for r in range(out.shape[0]):
+            if r not in touched:
+                assert_bit_equal(out[r], before[r], f"untouched row {r}")
+
+
+def test_destindex_copy_kv_is_raw_bytes():
+    # NaN payloads and negative zeros survive: the copy never goes through arithmetic
+    k = torch.tensor([[0x7E01, 0x8000, 0xFC00, 0x0001]], dtype=torch.int32).to(torch.int16).view(torch.float16).reshape(1, 1, 4)
+    out = torch.zeros(3, 1, 4, dtype=torch.float16)
+    O.destindex_copy_kv(k, torch.tensor([2]), out)
+    assert_bit_equal(out[2:3], k)
+
+
+# ----------------------------------------------------------------------------- token_attention
+def test_token_attention_window_fixture(golden):
+    fx = golden["token_attention"]
+    b_loc = torch.tensor(fx["b_loc"], dtype=torch.int32)
+    # independent statement of the window: the last L_i of the first max_input_len entries of row i
+    for i, (L, want) in enumerate(zip(fx["b_seq_len"], fx["expected_slots"])):
+        row = fx["b_loc"][i][: fx["max_input_len"]]
+        assert row[len(row) - L:] == want
+        assert O._window(b_loc, i, L, fx["max_input_len"]).tolist() == want
+    # k[slot] = slot everywhere, q = ones  =>  out[h, start+t] = slot * D / sqrt(D)
+    D = 128
+    k = torch.arange(100, dtype=torch.float64).reshape(100, 1, 1).expand(100, 32, D).contiguous()
+    q = torch.ones(3, 32, D, dtype=torch.float64)
+    out = torch.full((32, 13), -7.0, dtype=torch.float64)
+    O.token_attention(q, k, out, b_loc, torch.tensor(fx["b_start_loc"]), torch.tensor(fx["b_seq_len"]), fx["max_input_len"], exact=True)
+    flat = [s for w in fx["expected_slots"] for s in w]
+    assert_close(out, (torch.tensor(flat, dtype=torch.float64) * D / math.sqrt(D)).expand(32, 13), 1e-14, 0, "slot pattern")
+
+
+def _brute_token_attention(q, k, b_loc, b_start, b_len, max_len, cols):
+    B, H, D = q.shape
+    G = H // k.shape[1]
+    out = np.full((H, cols), np.nan)
+    qn, kn = q.double().numpy(), k.double().numpy()
+    for i in range(B):
+        L = int(b_len[i])
+        for t in range(L):
+            slot = int(b_loc[i, max_len - L + t])
+            for h in range(H):
+                out[h, int(b_start[i]) + t] = float(np.dot(qn[i, h], kn[slot, h // G])) / math.sqrt(D)
+    return torch.from_numpy(out)
+
+
+@pytest.mark.parametrize("G", [1, 4])
+def test_token_attention_brute_force_and_closed_forms(G):
+    g = rng(9)
+    B, Hkv, D, slots, N = 3, 2, 16, 40, 11
+    H = Hkv * G
+    q = torch.randn(B, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(slots, Hkv, D, generator=g, dtype=torch.float64)
+    b_len = torch.tensor([1, 7, 4])
+    b_start = torch.tensor([0, 1, 8])
+    max_len = 7
+    b_loc = torch.stack([torch.randperm(slots, generator=g)[:N] for _ in range(B)]).int()
+    out = torch.full((H, 12), float("nan"), dtype=torch.float64)
+    O.token_attention(q, k, out, b_loc, b_start, b_len, max_len, exact=True)
+    want = _brute_token_attention(q, k, b_loc, b_start, b_len, max_len, 12)
+    assert_close(out, want, 1e-13, 1e-14, "brute force")
+    # L = 1: a single dot product
+    s0 = int(b_loc[0, max_len - 1])
+    assert abs(float(out[0, 0]) - float(q[0, 0] @ k[s0, 0]) / math.sqrt(D)) < 1e-13
+    # k = q  =>  |q|^2 / sqrt(D)
+    kk = torch.zeros_like(k)
+    kk[5] = q[0, ::G]
+    loc = torch.full((1, 3), 5, dtype=torch.int32)
+    o2 = torch.zeros(H, 1, dtype=torch.float64)
+    O.token_attention(q[:1], kk, o2, loc, torch.tensor([0]), torch.tensor([1]), 3, exact=True)
+    assert abs(float(o2[0, 0]) - float((q[0, 0] ** 2).sum()) / math.sqrt(D)) < 1e-12
+
+
+# ----------------------------------------------------------------------------- token_softmax_reducev
+def test_softmax_reducev_closed_forms(golden):
+    fx = golden["token_attention"]
+    g = rng(10)
+    b_loc = torch.tensor(fx["b_loc"], dtype=torch.int32)
+    b_start, b_len = torch.tensor(fx["b_start_loc"]), torch.tensor(fx["b_seq_len"])
+    v = torch.randn(100, 32, 128, generator=g, dtype=torch.float64)
+    # constant logits => the mean of the gathered rows
+    out = torch.zeros(3, 32, 128, dtype=torch.float64)
+    O.token_softmax_reducev(torch.full((32, 13), 0.25, dtype=torch.float64), v, out, b_loc, b_start, b_len, 5, 10, exact=True)
+    for i, slots in enumerate(fx["expected_slots"]):
+        assert_close(out[i], v[slots].mean(0), 1e-13, 1e-14, f"mean of rows, sequence {i}")
+    # one dominant logit => that row
+    logits = torch.zeros(32, 13, dtype=torch.float64)
+    logits[:, 6] = 800.0  # column 6 = sequence 1, token 2 -> slot 5
+    O.token_softmax_reducev(logits, v, out, b_loc, b_start, b_len, 5, 10, exact=True)
+    assert_close(out[1], v[5], 1e-13, 0, "dominant logit")
+    # L = 1 => exactly the row, bit for bit, in 16-bit too
+    v16 = v.half()
+    o16 = torch.zeros(1, 32, 128, dtype=torch.float16)
+    O.token_softmax_reducev(torch.randn(32, 1, generator=g).half(), v16, o16, torch.tensor([[9, 9, 42]], dtype=torch.int32), torch.tensor([0]),
+                            torch.tensor([1]), 3, 0)
+    assert_bit_equal(o16[0], v16[42], "L = 1")
+
+
+@pytest.mark.parametrize("G", [1, 2])
+def test_softmax_reducev_brute_force(G):
+    g = rng(11)
+    B, Hkv, D, slots = 2, 3, 8, 30
+    H = Hkv * G
+    b_len, b_start, max_len = torch.tensor([5, 3]), torch.tensor([0, 5]), 6
+    b_loc = torch.stack([torch.randperm(slots, generator=g)[:9] for _ in range(B)]).int()
+    logits = torch.randn(H, 8, generator=g, dtype=torch.float64)
+    v = torch.randn(slots, Hkv, D, generator=g, dtype=torch.float64)
+    out = torch.zeros(B, H, D, dtype=torch.float64)
+    O.token_softmax_reducev(logits, v, out, b_loc, b_start, b_len, max_len, 0, exact=True)
+    for i in range(B):
+        L, s = int(b_len[i]), int(b_start[i])
+        for h in range(H):
+            x = logits[h, s:s + L].numpy()
+            p = np.exp(x - x.max())
+            p /= p.sum()
+            acc = np.zeros(D)
+            for t in range(L):
+                acc += p[t] * v[int(b_loc[i, max_len - L + t]), h // G].numpy()
+            assert np.allclose(out[i, h].numpy(), acc, rtol=1e-13, atol=1e-14)
+
+
+# ----------------------------------------------------------------------------- context_attention
+def _brute_context(q, k, v, start, L):
+    H, D = q.shape[1], q.shape[2]
+    out = np.zeros((L, H, D))
+    qn, kn, vn = (t.double().numpy() for t in (q, k, v))
+    for r in range(L):
+        for h in range(H):
+            s = np.array([np.dot(qn[start + r, h], kn[start + j, h]) for j in range(r + 1)]) / math.sqrt(D)
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            out[r, h] = sum(p[j] * vn[start + j, h] for j in range(r + 1))
+    return torch.from_numpy(out)
+
+
+def test_context_attention_reference_fixtures(golden):
+    g = rng(12)
+    for case in golden["context_attention"]["cases"][:3]:
+        T, H, D = case["shape"]
+        H = 4  # the head count does not interact with the segment logic; keep the brute force quick
+        q, k, v = (torch.randn(T, H, D, generator=g, dtype=torch.float64) for _ in range(3))
+        out = torch.full((T, H, D), 123.0, dtype=torch.float64)
+        bs, bl = torch.tensor(case["b_start_loc"]), torch.tensor(case["b_seq_len"])
+        O.context_attention(q, k, v, out, bs, bl, case["max_input_len"], exact=True)
+        covered = torch.zeros(T, dtype=torch.bool)
+        for s, L in zip(case["b_start_loc"], case["b_seq_len"]):
+            assert_close(out[s:s + L], _brute_context(q, k, v, s, L), 1e-12, 1e-13, f"segment at {s}")
+            assert_bit_equal(out[s], v[s], "first token of a sequence returns its own v row")
+            covered[s:s + L] = True
+        assert bool((out[~covered] == 123.0).all()), "rows outside every sequence are untouched"
+    # the last fixture leaves rows 192..255 untouched (64+64+128 rows used out of 256: starts 0, 64, 128)
+    last = golden["context_attention"]["cases"][3]
+    assert last["b_start_loc"][-1] + last["b_seq_len"][-1] == 256
+
+
+def test_context_attention_constant_v_and_decode_cross_check():
+    g = rng(13)
+    T, H, D = 24, 2, 16
+    q, k = (torch.randn(T, H, D, generator=g, dtype=torch.float64) for _ in range(2))
+    v = torch.randn(1, H, D, generator=g, dtype=torch.float64).expand(T, H, D).contiguous()
+    out = torch.zeros(T, H, D, dtype=torch.float64)
+    O.context_attention(q, k, v, out, torch.tensor([0, 10]), torch.tensor([10, 14]), exact=True)
+    assert_close(out, v, 1e-13, 1e-14, "constant V")
+    # last row of a sequence == decode attention of that row over the same K/V
+    v = torch.randn(T, H, D, generator=g, dtype=torch.float64)
+    O.context_attention(q, k, v, out, torch.tensor([0, 10]), torch.tensor([10, 14]), exact=True)
+    b_loc = torch.arange(10, 24, dtype=torch.int32).reshape(1, 14)
+    logits = torch.zeros(H, 14, dtype=torch.float64)
+    O.token_attention(q[23:24], k, logits, b_loc, torch.tensor([0]), torch.tensor([14]), 14, exact=True)
+    dec = torch.zeros(1, H, D, dtype=torch.float64)
+    O.token_softmax_reducev(logits, v, dec, b_loc, torch.tensor([0]), torch.tensor([14]), 14, 0, exact=True)
+    assert_close(dec[0], out[23], 1e-12, 1e-13, "prefill last row vs decode")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_context_attention_dtype_faithful_close_to_exact(dtype):
+    g = rng(14)
+    T, H, D = 48, 3, 32
+    q, k, v = ((torch.randn(T, H, D, generator=g) * 0.5).to(dtype) for _ in range(3))
+    bs, bl = torch.tensor([0, 16]), torch.tensor([16, 32])
+    out = torch.zeros(T, H, D, dtype=dtype)
+    O.context_attention(q, k, v, out, bs, bl)
+    ex = torch.zeros(T, H, D, dtype=torch.float64)
+    O.context_attention(q, k, v, ex, bs, bl, exact=True)
+    tol = 1e-2 if dtype == torch.float16 else 1e-5
+    assert_close(out, ex, tol, tol, "reference composition vs float64")
