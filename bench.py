@@ -1,0 +1,339 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 DIOPI LLaMA-inference operators on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only cfg3] [--no-cpu]
+
+A "step" is one pass of the decode hot path at the configured decode shape (fp16, batch 64,
+32 heads x 128, KV cache [131072, 32, 128], lengths ~U(512, 2048)): two diopiDestIndexCopyKV calls
+(new K rows, new V rows), diopiTokenAttentionInference and diopiTokenSoftmaxReduceVInference.
+`value` is decode tokens/s (batch / step time).  The same JSON line carries, under "ops", the
+achieved HBM GB/s (or TFLOP/s) and roofline fraction of every operator at every configured shape,
+each next to the CPU restatement of the reference timed on this box's host cores.
+
+Timing: inputs resident in HBM; W untimed warm-up steps; K timed steps bracketed by HIP events on the
+stream the kernels are launched on (and a device synchronisation on both sides).  Operators whose
+working set is near the 256 MB last-level cache rotate over three buffer sets.
+Algorithmic bytes / flops are the formulas in diopi_amd/workloads.py.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0    # dense fp16 / bf16
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,cfg3,cfg4,cfg5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every operator here is a single-device kernel and nothing in this build "
+              "uses a second GPU (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from diopi_amd import runtime as rt
+    from diopi_amd import workloads as W
+    from diopi_amd.runtime import Sizes, Tensor
+
+    if not torch.cuda.is_available() or rt.device_count() < 1:
+        print("bench.py needs a GPU: the operators have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    dev = "cuda:0"
+    impl = rt.libs().impl
+    ctx = rt.Context()
+    K, Wm = args.steps, args.warmup
+    only = set(x for x in args.only.split(",") if x)
+    cores = torch.get_num_threads()
+
+    def check(ret, what):
+        rt.check_returncode(ret, what)
+
+    def timed(step_fn, steps=K, warmup=Wm):
+        """Average milliseconds per call of step_fn(i), events on the context's stream."""
+        for i in range(warmup):
+            step_fn(i)
+        ctx.synchronize()
+        torch.cuda.synchronize()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(ctx)
+        for i in range(steps):
+            step_fn(i)
+        e1.record(ctx)
+        ms = e0.elapsed_ms(e1)
+        ctx.synchronize()
+        torch.cuda.synchronize()
+        return ms / steps
+
+    def cpu_time(fn, budget_s=3.0, min_reps=1, max_reps=5):
+        """Median seconds of fn() on the host after one warm-up, bounded by a time budget."""
+        fn()
+        ts = []
+        t_all = time.perf_counter()
+        while len(ts) < max_reps and (len(ts) < min_reps or time.perf_counter() - t_all < budget_s):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        ts.sort()
+        return ts[len(ts) // 2]
+
+    ops = []
+
+    def record(name, cfg, ms, work, bound, dtype, cpu=None, note=None):
+        e = dict(op=name, config=cfg, dtype=dtype, ms=round(ms, 5), bound=bound)
+        if bound == "hbm":
+            ach = work / (ms * 1e-3) / 1e9
+            e.update(bytes=int(work), achieved_GBs=round(ach, 1), frac=round(ach / HBM_PEAK_GBS, 4))
+        else:
+            ach = work / (ms * 1e-3) / 1e12
+            e.update(flops=int(work), achieved_TFLOPs=round(ach, 2), frac=round(ach / MFMA_PEAK_TFLOPS, 4))
+        if cpu is not None:
+            e["cpu"] = cpu
+        if note:
+            e["note"] = note
+        ops.append(e)
+        print("# " + json.dumps(e), file=sys.stderr, flush=True)
+        return e
+
+    from oracle import ref_ops as O  # the CPU baseline leg only
+
+    # ------------------------------------------------------------------ cfg1: RMSNorm fwd + bwd, fp32
+    if not only or "cfg1" in only:
+        sets = [W.cfg1(dev, seed=1 + s) for s in range(3)]
+        n1, n2 = sets[0]["n1"], sets[0]["n2"]
+        ns = Sizes((n2,))
+        hs = []
+        for s in sets:
+            s["out"] = torch.empty_like(s["x"])
+            s["inv"] = torch.empty(n1, dtype=torch.float32, device=dev)
+            s["gi"] = torch.empty_like(s["x"])
+            s["gw"] = torch.empty_like(s["weight"])
+            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "grad_out", "out", "inv", "gi", "gw")})
+
+        def fwd(i):
+            h = hs[i % 3]
+            check(impl.diopiRMSNorm(ctx.handle, h["out"].handle, h["inv"].handle, h["x"].handle, ns.c, h["weight"].handle, None, 1e-6), "diopiRMSNorm")
+
+        def bwd(i):
+            h = hs[i % 3]
+            check(impl.diopiRMSNormBackward(ctx.handle, h["gi"].handle, h["gw"].handle, None, h["grad_out"].handle, h["x"].handle, h["weight"].handle, None,
+                                            h["inv"].handle, ns.c, 1e-6), "diopiRMSNormBackward")
+            ctx.clear_tensors()
+
+        ms_f = timed(fwd)
+        ms_b = timed(bwd)
+        cpu_f = cpu_b = None
+        if not args.no_cpu:
+            xc, wc, gc = sets[0]["x"].cpu(), sets[0]["weight"].cpu(), sets[0]["grad_out"].cpu()
+            ic = sets[0]["inv"].cpu()
+            t = cpu_time(lambda: O.rms_norm(xc, (n2,), wc, None, 1e-6))
+            cpu_f = dict(seconds=round(t, 4), GBs=round(W.rmsnorm_fwd_bytes(n1, n2, 4) / t / 1e9, 2), cores=cores, sample="full shape")
+            t = cpu_time(lambda: O.rms_norm_backward(gc, xc, wc, ic, (n2,)))
+            cpu_b = dict(seconds=round(t, 4), GBs=round(W.rmsnorm_bwd_bytes(n1, n2, 4) / t / 1e9, 2), cores=cores, sample="full shape")
+        record("diopiRMSNorm", "cfg1 fp32 [8192,4096]", ms_f, W.rmsnorm_fwd_bytes(n1, n2, 4), "hbm", "f32", cpu_f)
+        record("diopiRMSNormBackward", "cfg1 fp32 [8192,4096]", ms_b, W.rmsnorm_bwd_bytes(n1, n2, 4), "hbm", "f32", cpu_b)
+        del sets, hs
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ cfg2: bf16 prologue
+    if not only or "cfg2" in only:
+        sets = [W.cfg2(dev, seed=2 + s) for s in range(3)]
+        T, H, D, n2 = sets[0]["T"], sets[0]["H"], sets[0]["D"], sets[0]["n2"]
+        ns = Sizes((n2,))
+        hs = []
+        for s in sets:
+            s["out"] = torch.empty_like(s["x"])
+            s["inv"] = torch.empty(T, dtype=torch.float32, device=dev)
+            s["qo"] = torch.empty_like(s["q"])
+            s["ko"] = torch.empty_like(s["k"])
+            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "out", "inv", "q", "k", "cos", "sin", "qo", "ko")})
+
+        def norm(i):
+            h = hs[i % 3]
+            check(impl.diopiRMSNorm(ctx.handle, h["out"].handle, h["inv"].handle, h["x"].handle, ns.c, h["weight"].handle, None, 1e-6), "diopiRMSNorm")
+
+        def rot(i):
+            h = hs[i % 3]
+            check(impl.diopiRotaryEmbedding(ctx.handle, h["qo"].handle, h["q"].handle, h["cos"].handle, h["sin"].handle, False, False), "diopiRotaryEmbedding")
+            check(impl.diopiRotaryEmbedding(ctx.handle, h["ko"].handle, h["k"].handle, h["cos"].handle, h["sin"].handle, False, False), "diopiRotaryEmbedding")
+
+        ms_n = timed(norm)
+        ms_r = timed(rot)
+        cpu_n = cpu_r = None
+        if not args.no_cpu:
+            xc, wc = sets[0]["x"].cpu(), sets[0]["weight"].cpu()
+            t = cpu_time(lambda: O.rms_norm(xc, (n2,), wc, None, 1e-6))
+            cpu_n = dict(seconds=round(t, 4), GBs=round(W.rmsnorm_fwd_bytes(T, n2, 2) / t / 1e9, 2), cores=cores, sample="full shape")
+            qc, cc, sc = sets[0]["q"].cpu(), sets[0]["cos"].cpu(), sets[0]["sin"].cpu()
+            t = cpu_time(lambda: O.rotary_emb(qc, cc, sc, False))
+            cpu_r = dict(seconds=round(2 * t, 4), GBs=round(W.rotary_bytes(T, H, D, 2) / t / 1e9, 2), cores=cores, sample="q call timed, k call assumed equal")
+        record("diopiRMSNorm", "cfg2 bf16 [16384,4096]", ms_n, W.rmsnorm_fwd_bytes(T, n2, 2), "hbm", "bf16", cpu_n)
+        record("diopiRotaryEmbedding x2 (q,k)", "cfg2 bf16 [16384,32,128]", ms_r, 2 * W.rotary_bytes(T, H, D, 2), "hbm", "bf16", cpu_r)
+        del sets, hs
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ decode configurations
+    def decode(w, tag, dtype_name):
+        e = 2
+        B, H, Hkv, D, total = w["B"], w["H"], w["Hkv"], w["D"], w["total_len"]
+        logits = torch.zeros(H, total, dtype=w["dtype"], device=dev)
+        out = torch.zeros_like(w["q"])
+        h = {k: Tensor(w[k]) for k in ("k_cache", "v_cache", "q", "new_k", "new_v", "dest_loc", "b_loc", "b_seq_len", "b_start_loc")}
+        h["logits"], h["out"] = Tensor(logits), Tensor(out)
+        mil = w["max_input_len"]
+
+        def copy_kv(i):
+            check(impl.diopiDestIndexCopyKV(ctx.handle, h["k_cache"].handle, h["new_k"].handle, h["dest_loc"].handle), "diopiDestIndexCopyKV")
+            check(impl.diopiDestIndexCopyKV(ctx.handle, h["v_cache"].handle, h["new_v"].handle, h["dest_loc"].handle), "diopiDestIndexCopyKV")
+
+        def att(i):
+            check(impl.diopiTokenAttentionInference(ctx.handle, h["logits"].handle, h["q"].handle, h["k_cache"].handle, h["b_loc"].handle,
+                                                    h["b_start_loc"].handle, h["b_seq_len"].handle, mil), "diopiTokenAttentionInference")
+
+        def redv(i):
+            check(impl.diopiTokenSoftmaxReduceVInference(ctx.handle, h["out"].handle, h["logits"].handle, h["v_cache"].handle, h["b_loc"].handle,
+                                                         h["b_start_loc"].handle, h["b_seq_len"].handle, mil, 0), "diopiTokenSoftmaxReduceVInference")
+            ctx.clear_tensors()
+
+        def step(i):
+            copy_kv(i)
+            att(i)
+            redv(i)
+
+        ms_copy = timed(copy_kv)
+        ms_att = timed(att)
+        ms_red = timed(redv)
+        ms_step = timed(step)
+        b_att = W.token_attention_bytes(total, B, H, Hkv, D, e)
+        b_red = W.softmax_reducev_bytes(total, B, H, Hkv, D, e)
+        b_copy = 2 * W.destindex_bytes(B, Hkv, D, e)
+        cpu = None
+        if not args.no_cpu:
+            # bounded sample: the first sequences of the batch through the reference's per-sequence composition
+            qc, blc, bsc, bln = w["q"].cpu(), w["b_loc"].cpu(), w["b_start_loc"].cpu(), w["b_seq_len"].cpu()
+            nseq, spent, tok = 0, 0.0, 0
+            budget = args.cpu_seconds if tag == "cfg3" else 4.0
+            while nseq < B and spent < budget:
+                sel = slice(nseq, nseq + 1)
+                used = torch.unique(blc[sel].long())
+                remap = torch.zeros(int(used.max()) + 1, dtype=torch.int32)
+                remap[used] = torch.arange(used.numel(), dtype=torch.int32)
+                ks, vs = w["k_cache"][used.to(dev)].cpu(), w["v_cache"][used.to(dev)].cpu()
+                loc = remap[blc[sel].long()]
+                lg = torch.zeros(H, total, dtype=w["dtype"])
+                oc = torch.zeros(1, H, D, dtype=w["dtype"])
+                t0 = time.perf_counter()
+                O.token_attention(qc[sel], ks, lg, loc, bsc[sel], bln[sel], mil)
+                O.token_softmax_reducev(lg, vs, oc, loc, bsc[sel], bln[sel], mil, 0)
+                spent += time.perf_counter() - t0
+                tok += int(bln[nseq])
+                nseq += 1
+            frac_tok = tok / total
+            cpu = dict(seconds_sample=round(spent, 3), sequences=nseq, tokens_per_s=round(nseq / spent, 2),
+                       GBs=round((b_att + b_red) * frac_tok / spent / 1e9, 3), cores=cores,
+                       sample=f"first {nseq} of {B} sequences ({tok} of {total} cached tokens), attention only, cache rows pre-gathered")
+        record("diopiDestIndexCopyKV x2 (K,V)", f"{tag} {B} tokens", ms_copy, b_copy, "hbm", dtype_name,
+               note="launch-bound at this size: 1 MiB of traffic per call")
+        record("diopiTokenAttentionInference", tag, ms_att, b_att, "hbm", dtype_name)
+        record("diopiTokenSoftmaxReduceVInference", tag, ms_red, b_red, "hbm", dtype_name)
+        e_step = record("decode step (copy K,V + attention)", tag, ms_step, b_copy + b_att + b_red, "hbm", dtype_name, cpu)
+        e_step["tokens_per_s"] = round(B / (ms_step * 1e-3), 1)
+        e_step["attention_only_tokens_per_s"] = round(B / ((ms_att + ms_red) * 1e-3), 1)
+        return dict(ms_step=ms_step, ms_att=ms_att, ms_red=ms_red, b_att=b_att, b_red=b_red, B=B, total=total, cpu=cpu)
+
+    head = None
+    if not only or "cfg3" in only:
+        w3 = W.cfg3(dev, seed=3)
+        head = decode(w3, "cfg3", "f16")
+        # DestIndexCopyKV away from the launch-bound regime: a full permutation of 65536 rows of 8 KiB
+        Tn = 65536
+        src = w3["k_cache"][:Tn].clone()
+        perm = torch.randperm(Tn, device=dev).int() + Tn
+        hsrc, hperm, hcache = Tensor(src), Tensor(perm), Tensor(w3["k_cache"])
+        ms = timed(lambda i: check(impl.diopiDestIndexCopyKV(ctx.handle, hcache.handle, hsrc.handle, hperm.handle), "diopiDestIndexCopyKV"))
+        record("diopiDestIndexCopyKV", f"sweep: {Tn} tokens x 8 KiB", ms, W.destindex_bytes(Tn, 32, 128, 2), "hbm", "f16")
+        del w3, src, perm, hsrc, hperm, hcache
+        torch.cuda.empty_cache()
+
+    if not only or "cfg5" in only:
+        w5 = W.cfg5(dev, seed=5)
+        decode(w5, "cfg5", "bf16")
+        del w5
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ cfg4: prefill
+    if not only or "cfg4" in only:
+        w4 = W.cfg4(dev, seed=4)
+        out = torch.zeros_like(w4["q"])
+        h = {k: Tensor(w4[k]) for k in ("q", "k", "v", "b_start_loc", "b_seq_len")}
+        h["out"] = Tensor(out)
+        flops = W.context_attention_flops(w4["seq_len_host"], w4["H"], w4["D"])
+
+        def pre(i):
+            check(impl.diopiContextAttentionInference(ctx.handle, h["out"].handle, h["q"].handle, h["k"].handle, h["v"].handle, h["b_start_loc"].handle,
+                                                      h["b_seq_len"].handle, w4["max_input_len"]), "diopiContextAttentionInference")
+
+        ms = timed(pre, steps=max(5, K // 5), warmup=max(2, Wm // 5))
+        cpu = None
+        if not args.no_cpu:
+            # the reference materialises [H, L, L] scores and ATen's fp16 matmul on the host is slow: time the first
+            # 256 rows of the shortest sequence only and scale by flops
+            i = int(w4["seq_len_host"].argmin())
+            s, L = int(w4["b_start_loc"][i]), min(256, int(w4["seq_len_host"][i]))
+            qc, kc, vc = (w4[k][s:s + L].cpu() for k in ("q", "k", "v"))
+            oc = torch.zeros_like(qc)
+            t0 = time.perf_counter()
+            O.context_attention(qc, kc, vc, oc, torch.tensor([0]), torch.tensor([L]), L)
+            t = time.perf_counter() - t0
+            f1 = W.context_attention_flops([L], w4["H"], w4["D"])
+            cpu = dict(seconds_sample=round(t, 3), TFLOPs=round(f1 / t / 1e12, 4), cores=cores,
+                       sample=f"first {L} rows of the shortest sequence; extrapolated by flops to the full configuration: {t * flops / f1:.1f} s")
+        record("diopiContextAttentionInference", f"cfg4 fp16 B=8 T={w4['T']}", ms, flops, "mfma", "f16", cpu)
+        del w4
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ the JSON line
+    line = {
+        "metric": "decode-attn tokens/s at bs=64 (per-op achieved HBM GB/s and % of peak under 'ops')",
+        "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "cfg3 decode step fp16: 2x DestIndexCopyKV [64,32,128] -> cache [131072,32,128], TokenAttention + "
+                               "TokenSoftmaxReduceV, batch 64, 32 heads x 128, b_loc [64,2048], seq_len ~U(512,2048)"},
+        "roofline": None, "cpu_baseline": None, "ops": ops,
+        "peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_TFLOPs": MFMA_PEAK_TFLOPS},
+    }
+    if head is not None:
+        line["value"] = round(head["B"] / (head["ms_step"] * 1e-3), 1)
+        line["ms_per_step"] = round(head["ms_step"], 5)
+        line["config"]["total_cached_tokens"] = head["total"]
+        # dominant kernel of the step: the slower of the two attention halves
+        if head["ms_att"] >= head["ms_red"]:
+            kname, kms, kbytes = "tokenAttMfma (diopiTokenAttentionInference)", head["ms_att"], head["b_att"]
+        else:
+            kname, kms, kbytes = "softmaxReduceVSplit+Merge (diopiTokenSoftmaxReduceVInference)", head["ms_red"], head["b_red"]
+        ach = kbytes / (kms * 1e-3) / 1e9
+        line["roofline"] = {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}
+        if head["cpu"] is not None:
+            c = head["cpu"]
+            line["cpu_baseline"] = {"value": c["tokens_per_s"], "unit": "tokens/s", "cores": c["cores"], "kind": "port", "sample": c["sample"]}
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -252,6 +252,13 @@ const DeviceInfo& deviceInfo() {
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) {
             d.numCU = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : d.numCU;
             d.maxSharedPerBlock = static_cast<int>(prop.sharedMemPerBlock);
+            int optin = 0;
+            if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, dev) == hipSuccess && optin > 0) {
+                d.maxSharedOptin = optin;
+            } else {
+                (void)hipGetLastError();
+                d.maxSharedOptin = d.maxSharedPerBlock;
+            }
         } else {
             (void)hipGetLastError();
         }

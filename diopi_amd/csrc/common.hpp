@@ -112,6 +112,7 @@ diopiError_t zeroFill(hipStream_t stream, void* ptr, int64_t bytes);
 struct DeviceInfo {
     int numCU = 256;
     int maxSharedPerBlock = 65536;
+    int maxSharedOptin = 65536;  // LDS a work-group may use with dynamic shared memory granted explicitly
 };
 const DeviceInfo& deviceInfo();
 

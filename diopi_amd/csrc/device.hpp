@@ -111,6 +111,21 @@ __device__ __forceinline__ T waveMax(T v) {
     return v;
 }
 
+// v_mfma_f32_16x16x32 on 16-bit operands: lane l supplies row/column l % 16 and the 8 consecutive k
+// values 8 * (l / 16) .. +7 of A and of B; it receives rows 4 * (l / 16) .. +3 of column l % 16 of C.
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<half_t> {
+    using Frag = f16x8;
+    static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+template <>
+struct Mfma16<bf16_t> {
+    using Frag = bf16x8;
+    static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+
 // Reads an index tensor element as int64 whatever its storage width.
 __device__ __forceinline__ int64_t loadIndex(const void* base, int64_t i, bool is64) {
     return is64 ? reinterpret_cast<const int64_t*>(base)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(base)[i]);

@@ -121,6 +121,107 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdRowReg(TOut* __restrict
 }
 
 // ---------------------------------------------------------------------------
+// Forward for long rows (more than two packets per lane of a wave): a 256-thread group owns a row, each
+// thread NVT packets of it; the sum of squares crosses the four waves through LDS (one barrier per
+// row).  Many short-lived groups, each touching one contiguous run of rows, is the launch shape the
+// memory system sustains the highest bandwidth for.
+// ---------------------------------------------------------------------------
+template <typename TIn, typename TOut, int NVT, bool HAS_BIAS>
+__global__ __launch_bounds__(kFwdThreads) void rmsNormFwdBlockRow(TOut* __restrict__ out, float* __restrict__ invRms, const TIn* __restrict__ x,
+                                                                   const TOut* __restrict__ weight, const TOut* __restrict__ bias, int64_t n1, int n2,
+                                                                   float eps, int rowsPerBlock) {
+    constexpr int EPV = Pack16<TIn>::N;
+    __shared__ float red[2][kFwdWaves];
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int nvec = n2 / EPV;
+    int64_t row = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
+    int64_t rowEnd = row + rowsPerBlock;
+    if (rowEnd > n1) rowEnd = n1;
+
+    float w[NVT][EPV];
+    float b[NVT][EPV];
+#pragma unroll
+    for (int j = 0; j < NVT; ++j) {
+        const int v = j * kFwdThreads + tid;
+        if (v < nvec) {
+            if constexpr (sizeof(TOut) == sizeof(TIn)) {
+                const Pack16<TOut> wp = loadPack(weight + v * EPV);
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) w[j][e] = toFloat(wp.e[e]);
+                if (HAS_BIAS) {
+                    const Pack16<TOut> bp = loadPack(bias + v * EPV);
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) b[j][e] = toFloat(bp.e[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    w[j][e] = toFloat(weight[v * EPV + e]);
+                    if (HAS_BIAS) b[j][e] = toFloat(bias[v * EPV + e]);
+                }
+            }
+        }
+    }
+    const float rn2 = 1.0f / static_cast<float>(n2);
+    int parity = 0;
+    for (; row < rowEnd; ++row, parity ^= 1) {
+        const TIn* xr = x + row * n2;
+        TOut* orow = out + row * n2;
+        Pack16<TIn> xv[NVT];
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kFwdThreads + tid;
+            if (v < nvec) xv[j] = loadPackStream(xr + v * EPV);
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kFwdThreads + tid;
+            if (v < nvec) {
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const float f = toFloat(xv[j].e[e]);
+                    ss += f * f;
+                }
+            }
+        }
+        ss = waveSum(ss);
+        if (lane == 0) red[parity][wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < kFwdWaves; ++i) tot += red[parity][i];
+        const float inv = 1.0f / sqrtf(tot * rn2 + eps);
+        if (tid == 0) invRms[row] = inv;
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            const int v = j * kFwdThreads + tid;
+            if (v < nvec) {
+                TOut o[EPV];
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) {
+                    const TOut normed = fromFloat<TOut>(inv * toFloat(xv[j].e[e]));
+                    TOut r = fromFloat<TOut>(w[j][e] * toFloat(normed));
+                    if (HAS_BIAS) r = fromFloat<TOut>(toFloat(r) + b[j][e]);
+                    o[e] = r;
+                }
+                if constexpr (sizeof(TOut) == sizeof(TIn)) {
+                    Pack16<TOut> pv;
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) pv.e[e] = o[e];
+                    storePackStream(orow + v * EPV, pv);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) orow[v * EPV + e] = o[e];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Forward, any shape / dtype combination: one wavefront per row, two sweeps over the row
 // (the second one hits in cache).  AccT is float or double.
 // ---------------------------------------------------------------------------
@@ -158,112 +259,152 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 
 // ---------------------------------------------------------------------------
 // Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
-// Thread t of a 256-thread group owns packets t, t+256, ... of every row.
+// A work-group is GROUPS row teams of 256 threads; team g takes rows row0+g, row0+g+GROUPS, ...
+// Thread t of a team owns packets t, t+256, ... of every row its team visits.  The column sums for
+// grad_weight / grad_bias live in LDS, one private array per team (ds_add, no return value needed), which
+// keeps them out of the register file: the registers hold the current row and the prefetched next row
+// instead, so loads stay in flight across the one barrier per row step (the row sum s[r] crosses the
+// team's four waves through LDS).  At the end the team arrays are summed in a fixed order into one
+// partial row per work-group.  One large work-group per compute unit keeps the partial buffer at one
+// row per unit while 16 waves keep enough loads in flight.
 // ---------------------------------------------------------------------------
-constexpr int kBwdThreads = 256;
-constexpr int kBwdWaves = kBwdThreads / kWave;
+constexpr int kBwdTeam = 256;
+constexpr int kBwdTeamWaves = kBwdTeam / kWave;
 
-template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS>
-__global__ __launch_bounds__(kBwdThreads) void rmsNormBwdFused(T* __restrict__ gradInput, ColAcc* __restrict__ partW, ColAcc* __restrict__ partB,
-                                                                const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
-                                                                const float* __restrict__ invRms, int64_t n1, int n2, int rowsPerBlock) {
+template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS>
+__global__ __launch_bounds__(kBwdTeam* GROUPS) void rmsNormBwdFused(T* __restrict__ gradInput, ColAcc* __restrict__ partW, ColAcc* __restrict__ partB,
+                                                                       const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
+                                                                       const float* __restrict__ invRms, int64_t n1, int n2, int rowsPerBlock) {
     constexpr int EPV = Pack16<T>::N;
-    __shared__ float red[2][kBwdWaves];
-    const int tid = threadIdx.x;
+    constexpr int kCols = NVT * kBwdTeam * EPV;  // columns covered by the register tiling
+    __shared__ float red[2][GROUPS][kBwdTeamWaves];
+    extern __shared__ __attribute__((aligned(16))) unsigned char dynLds[];
+    // [array(W,B)][team][(j*EPV + e)][tid]: lanes of a wave hit consecutive words
+    ColAcc* sAcc = reinterpret_cast<ColAcc*>(dynLds);
+    const int team = threadIdx.x / kBwdTeam;
+    const int tid = threadIdx.x % kBwdTeam;
     const int lane = tid % kWave;
     const int wave = tid / kWave;
     const int nvec = n2 / EPV;
+    ColAcc* myW = sAcc + team * kCols;
+    ColAcc* myB = sAcc + (GROUPS + team) * kCols;
 
     float w[NVT][EPV];
-    ColAcc accW[NVT][EPV];
-    ColAcc accB[NVT][EPV];
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-        const int v = j * kBwdThreads + tid;
+        const int v = j * kBwdTeam + tid;
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
-            accW[j][e] = 0;
-            accB[j][e] = 0;
             w[j][e] = (v < nvec) ? toFloat(weight[v * EPV + e]) : 0.f;
+            myW[(j * EPV + e) * kBwdTeam + tid] = 0;
+            if (HAS_GBIAS) myB[(j * EPV + e) * kBwdTeam + tid] = 0;
         }
     }
 
-    int64_t row = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
-    int64_t rowEnd = row + rowsPerBlock;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
+    int64_t rowEnd = row0 + rowsPerBlock;
     if (rowEnd > n1) rowEnd = n1;
     const float fH = static_cast<float>(n2);
     int parity = 0;
-    for (; row < rowEnd; ++row, parity ^= 1) {
-        const T* xr = x + row * n2;
-        const T* dr = dout + row * n2;
-        Pack16<T> xv[NVT], dv[NVT];
+    // The rows of the next step are requested before the current step is reduced and written back.
+    Pack16<T> xv[NVT], dv[NVT], xn[NVT], dn[NVT];
+    float inv = 0.f, invNext = 0.f;
+    auto request = [&](int64_t row, Pack16<T>* xb, Pack16<T>* db, float* invp) {
+        if (row < rowEnd) {
+            const T* xr = x + row * n2;
+            const T* dr = dout + row * n2;
 #pragma unroll
-        for (int j = 0; j < NVT; ++j) {
-            const int v = j * kBwdThreads + tid;
-            if (v < nvec) {
-                xv[j] = loadPackStream(xr + v * EPV);
-                dv[j] = loadPackStream(dr + v * EPV);
+            for (int j = 0; j < NVT; ++j) {
+                const int v = j * kBwdTeam + tid;
+                if (v < nvec) {
+                    xb[j] = loadPackStream(xr + v * EPV);
+                    db[j] = loadPackStream(dr + v * EPV);
+                }
             }
+            *invp = invRms[row];
         }
-        const float inv = invRms[row];
+    };
+    request(row0 + team, xv, dv, &inv);
+    // every team runs the same number of steps so that the barrier below is reached by all of them
+    for (int64_t base = row0; base < rowEnd; base += GROUPS, parity ^= 1) {
+        const int64_t row = base + team;
+        const bool live = row < rowEnd;
+        request(row + GROUPS, xn, dn, &invNext);
         float s = 0.f;
+        if (live) {
 #pragma unroll
-        for (int j = 0; j < NVT; ++j) {
-            const int v = j * kBwdThreads + tid;
-            if (v < nvec) {
+            for (int j = 0; j < NVT; ++j) {
+                const int v = j * kBwdTeam + tid;
+                if (v < nvec) {
 #pragma unroll
-                for (int e = 0; e < EPV; ++e) {
-                    const float cx = toFloat(xv[j].e[e]);
-                    const float cd = toFloat(dv[j].e[e]);
-                    s += cd * w[j][e] * cx * inv;
-                    accW[j][e] += static_cast<ColAcc>(cd * cx * inv);
-                    if (HAS_GBIAS) accB[j][e] += static_cast<ColAcc>(cd);
+                    for (int e = 0; e < EPV; ++e) {
+                        const float cx = toFloat(xv[j].e[e]);
+                        const float cd = toFloat(dv[j].e[e]);
+                        s += cd * w[j][e] * cx * inv;
+                        // each (team, column) word has exactly one writer: the add is a plain read-modify-write done by the LDS unit
+                        atomicAdd(&myW[(j * EPV + e) * kBwdTeam + tid], static_cast<ColAcc>(cd * cx * inv));
+                        if (HAS_GBIAS) atomicAdd(&myB[(j * EPV + e) * kBwdTeam + tid], static_cast<ColAcc>(cd));
+                    }
                 }
             }
         }
         s = waveSum(s);
-        if (lane == 0) red[parity][wave] = s;
+        if (lane == 0) red[parity][team][wave] = s;
         __syncthreads();
-        float sum2 = 0.f;
+        if (live) {
+            float sum2 = 0.f;
 #pragma unroll
-        for (int i = 0; i < kBwdWaves; ++i) sum2 += red[parity][i];
-        const float term1 = (1.0f / fH) * inv;
-        T* gr = gradInput + row * n2;
+            for (int i = 0; i < kBwdTeamWaves; ++i) sum2 += red[parity][team][i];
+            const float term1 = (1.0f / fH) * inv;
+            T* gr = gradInput + row * n2;
 #pragma unroll
-        for (int j = 0; j < NVT; ++j) {
-            const int v = j * kBwdThreads + tid;
-            if (v < nvec) {
-                Pack16<T> gv;
+            for (int j = 0; j < NVT; ++j) {
+                const int v = j * kBwdTeam + tid;
+                if (v < nvec) {
+                    Pack16<T> gv;
 #pragma unroll
-                for (int e = 0; e < EPV; ++e) {
-                    const float cx = toFloat(xv[j].e[e]);
-                    const float cd = toFloat(dv[j].e[e]);
-                    float f = fH * cd * w[j][e];
-                    f -= cx * inv * sum2;
-                    f *= term1;
-                    gv.e[e] = fromFloat<T>(f);
+                    for (int e = 0; e < EPV; ++e) {
+                        const float cx = toFloat(xv[j].e[e]);
+                        const float cd = toFloat(dv[j].e[e]);
+                        float f = fH * cd * w[j][e];
+                        f -= cx * inv * sum2;
+                        f *= term1;
+                        gv.e[e] = fromFloat<T>(f);
+                    }
+                    storePackStream(gr + v * EPV, gv);
                 }
-                storePackStream(gr + v * EPV, gv);
             }
         }
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+            xv[j].raw = xn[j].raw;
+            dv[j].raw = dn[j].raw;
+        }
+        inv = invNext;
     }
 
-    // this group's column partials
+    // one partial row per work-group: the team arrays are added in team order
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < kCols; idx += kBwdTeam * GROUPS) {
+        // idx = (j*EPV + e)*256 + t  <->  column (j*256 + t)*EPV + e
+        const int t = idx % kBwdTeam;
+        const int je = idx / kBwdTeam;
+        const int col = ((je / EPV) * kBwdTeam + t) * EPV + (je % EPV);
+        if (col < n2) {
+            ColAcc sw = 0, sb = 0;
 #pragma unroll
-    for (int j = 0; j < NVT; ++j) {
-        const int v = j * kBwdThreads + tid;
-        if (v < nvec) {
-#pragma unroll
-            for (int e = 0; e < EPV; ++e) {
-                partW[static_cast<int64_t>(blockIdx.x) * n2 + v * EPV + e] = accW[j][e];
-                if (HAS_GBIAS) partB[static_cast<int64_t>(blockIdx.x) * n2 + v * EPV + e] = accB[j][e];
+            for (int g = 0; g < GROUPS; ++g) {
+                sw += sAcc[g * kCols + idx];
+                if (HAS_GBIAS) sb += sAcc[(GROUPS + g) * kCols + idx];
             }
+            partW[static_cast<int64_t>(blockIdx.x) * n2 + col] = sw;
+            if (HAS_GBIAS) partB[static_cast<int64_t>(blockIdx.x) * n2 + col] = sb;
         }
     }
 }
 
-// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias).  A 256-thread group covers
-// 64 columns x 4 row slices; lanes of a wave read consecutive columns.
+// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias) in fp64.  A 256-thread group
+// covers 64 columns x 4 slices of the partial rows; lanes of a wave read consecutive columns.
 template <typename T, typename ColAcc>
 __global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight, T* __restrict__ gradBias, const ColAcc* __restrict__ partW,
                                                        const ColAcc* __restrict__ partB, int numParts, int n2) {
@@ -273,9 +414,20 @@ __global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight
     const int col = blockIdx.x * 64 + lane;
     double sw = 0.0, sb = 0.0;
     if (col < n2) {
-        for (int p = slice; p < numParts; p += 4) {
-            sw += static_cast<double>(partW[static_cast<int64_t>(p) * n2 + col]);
-            if (gradBias != nullptr) sb += static_cast<double>(partB[static_cast<int64_t>(p) * n2 + col]);
+        constexpr int kBatch = 8;  // loads of a batch are independent and in flight together
+        for (int p0 = slice; p0 < numParts; p0 += 4 * kBatch) {
+            ColAcc vw[kBatch], vb[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int p = p0 + 4 * u;
+                vw[u] = p < numParts ? partW[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
+                vb[u] = (gradBias != nullptr && p < numParts) ? partB[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                sw += static_cast<double>(vw[u]);
+                sb += static_cast<double>(vb[u]);
+            }
         }
     }
     red[0][slice][lane] = sw;
@@ -376,14 +528,42 @@ diopiError_t launchFwdFast(hipStream_t stream, const TensorView& out, const Tens
     if (nvec > 16 * kWave) return diopiSuccess;
     if (!aligned16(in.data) || !aligned16(out.data) || !aligned16(w.data)) return diopiSuccess;
     if (sizeof(TOut) != sizeof(TIn) && (reinterpret_cast<uintptr_t>(out.data) & 7) != 0) return diopiSuccess;
+    const float feps = static_cast<float>(eps);
+    const int n2 = static_cast<int>(d.n2);
+    if (nvec > 2 * kWave && envInt("DIOPI_ROCM_RMSFWD_WAVEROW", 0) == 0) {
+        // long rows: one 256-thread group per run of rows
+        const int nvt = static_cast<int>(ceilDiv(nvec, kFwdThreads));
+        int rpb = envInt("DIOPI_ROCM_RMSFWD_ROWS_PER_BLOCK", 1);
+        if (rpb < 1) rpb = 1;
+        const unsigned gridB = static_cast<unsigned>(ceilDiv(d.n1, rpb));
+#define ROCM_FWDB_CASE(NVC)                                                                                                                         \
+    if (bias != nullptr) {                                                                                                                          \
+        hipLaunchKernelGGL((rmsNormFwdBlockRow<TIn, TOut, NVC, true>), dim3(gridB), dim3(kFwdThreads), 0, stream, static_cast<TOut*>(out.data),      \
+                           static_cast<float*>(invRms.data), static_cast<const TIn*>(in.data), static_cast<const TOut*>(w.data),                      \
+                           static_cast<const TOut*>(bias), d.n1, n2, feps, rpb);                                                                      \
+    } else {                                                                                                                                        \
+        hipLaunchKernelGGL((rmsNormFwdBlockRow<TIn, TOut, NVC, false>), dim3(gridB), dim3(kFwdThreads), 0, stream, static_cast<TOut*>(out.data),     \
+                           static_cast<float*>(invRms.data), static_cast<const TIn*>(in.data), static_cast<const TOut*>(w.data),                      \
+                           static_cast<const TOut*>(nullptr), d.n1, n2, feps, rpb);                                                                   \
+    }
+        if (nvt <= 1) {
+            ROCM_FWDB_CASE(1)
+        } else if (nvt <= 2) {
+            ROCM_FWDB_CASE(2)
+        } else {
+            ROCM_FWDB_CASE(4)
+        }
+#undef ROCM_FWDB_CASE
+        ROCM_LAUNCH_CHECK();
+        *launched = true;
+        return diopiSuccess;
+    }
     const int nv = static_cast<int>(ceilDiv(nvec, kWave));
     // every wave takes the same number of rows so that all of them fit on the device at once
     int rowsPerWave = static_cast<int>(ceilDiv(d.n1, residentWavesTarget()));
     if (rowsPerWave < 1) rowsPerWave = 1;
     const int64_t waves = ceilDiv(d.n1, rowsPerWave);
     const unsigned grid = static_cast<unsigned>(ceilDiv(waves, kFwdWaves));
-    const float feps = static_cast<float>(eps);
-    const int n2 = static_cast<int>(d.n2);
 #define ROCM_FWD_CASE(NVC)                                                                                                                          \
     if (bias != nullptr) {                                                                                                                          \
         hipLaunchKernelGGL((rmsNormFwdRowReg<TIn, TOut, NVC, true>), dim3(grid), dim3(kFwdThreads), 0, stream, static_cast<TOut*>(out.data),         \
@@ -436,6 +616,22 @@ diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const Tenso
     return launchFwdGeneric<TIn, TOut, AccT>(stream, out, invRms, in, w, bias, d, eps);
 }
 
+// Launches one instantiation of the fused backward kernel; the LDS column-sum arrays are dynamic shared memory
+// beyond the 64 KiB static limit, which has to be granted per kernel once.
+template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS>
+diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, ColAcc* partW, ColAcc* partB, const T* dout, const T* in, const T* w,
+                               const float* invRms, int64_t n1, int n2, int rowsPerBlock) {
+    constexpr int EPV = Pack16<T>::N;
+    constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * kBwdTeam * EPV * sizeof(ColAcc);
+    auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS>;
+    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                    static_cast<int>(ldsBytes));
+    ROCM_HIP(granted);
+    hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2, rowsPerBlock);
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
 template <typename T, typename ColAcc>
 diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& gIn, const TensorView& gW, void* gBias, const TensorView& dout,
                             const TensorView& in, const TensorView& w, const TensorView& invRms, const NormDims& d, bool* launched) {
@@ -443,12 +639,17 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     *launched = false;
     if (d.n2 % EPV != 0 || d.n2 > INT32_MAX) return diopiSuccess;
     const int64_t nvec = d.n2 / EPV;
-    if (nvec > 4 * kBwdThreads) return diopiSuccess;
+    // one team array is at most 32 KiB of LDS; four teams without grad_bias, two with (128 KiB per work-group)
+    constexpr int kMaxNvt = static_cast<int>(32768 / (kBwdTeam * EPV * sizeof(ColAcc)));
+    if (nvec > static_cast<int64_t>(kMaxNvt) * kBwdTeam) return diopiSuccess;
+    if (deviceInfo().maxSharedOptin < 128 * 1024 + 1024) return diopiSuccess;
     if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
-    const int nvt = static_cast<int>(ceilDiv(nvec, kBwdThreads));
-    int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * envInt("DIOPI_ROCM_RMSBWD_BLOCKS_PER_CU", 4);
-    int rowsPerBlock = static_cast<int>(ceilDiv(d.n1, maxBlocks));
-    if (rowsPerBlock < 1) rowsPerBlock = 1;
+    const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
+    const int groups = gBias ? 2 : 4;
+    // one work-group per compute unit, each walking a contiguous run of rows
+    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * envInt("DIOPI_ROCM_RMSBWD_BLOCKS_PER_CU", 1);
+    int64_t rowsPerBlock = ceilDiv(d.n1, maxBlocks);
+    rowsPerBlock = ceilDiv(rowsPerBlock, groups) * groups;
     const int numParts = static_cast<int>(ceilDiv(d.n1, rowsPerBlock));
     const int n2 = static_cast<int>(d.n2);
     const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(ColAcc);
@@ -456,15 +657,19 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     ROCM_CALL(requireScratch(ctx, partBytes * (gBias ? 2 : 1), &scratch));
     ColAcc* partW = static_cast<ColAcc*>(scratch);
     ColAcc* partB = gBias ? partW + static_cast<int64_t>(numParts) * n2 : nullptr;
-#define ROCM_BWD_CASE(NVC)                                                                                                                             \
-    if (gBias != nullptr) {                                                                                                                            \
-        hipLaunchKernelGGL((rmsNormBwdFused<T, ColAcc, NVC, true>), dim3(numParts), dim3(kBwdThreads), 0, stream, static_cast<T*>(gIn.data), partW,     \
-                           partB, static_cast<const T*>(dout.data), static_cast<const T*>(in.data), static_cast<const T*>(w.data),                      \
-                           static_cast<const float*>(invRms.data), d.n1, n2, rowsPerBlock);                                                             \
-    } else {                                                                                                                                           \
-        hipLaunchKernelGGL((rmsNormBwdFused<T, ColAcc, NVC, false>), dim3(numParts), dim3(kBwdThreads), 0, stream, static_cast<T*>(gIn.data), partW,    \
-                           partB, static_cast<const T*>(dout.data), static_cast<const T*>(in.data), static_cast<const T*>(w.data),                      \
-                           static_cast<const float*>(invRms.data), d.n1, n2, rowsPerBlock);                                                             \
+    const int rpb = static_cast<int>(rowsPerBlock);
+    T* pgi = static_cast<T*>(gIn.data);
+    const T* pdo = static_cast<const T*>(dout.data);
+    const T* pin = static_cast<const T*>(in.data);
+    const T* pw = static_cast<const T*>(w.data);
+    const float* pinv = static_cast<const float*>(invRms.data);
+#define ROCM_BWD_CASE(NVC)                                                                                                          \
+    if constexpr (NVC <= kMaxNvt) {                                                                                                 \
+        if (gBias != nullptr) {                                                                                                     \
+            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, true, 2>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2, rpb)));  \
+        } else {                                                                                                                    \
+            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, false, 4>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2, rpb))); \
+        }                                                                                                                           \
     }
     if (nvt <= 1) {
         ROCM_BWD_CASE(1)
@@ -474,7 +679,6 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
         ROCM_BWD_CASE(4)
     }
 #undef ROCM_BWD_CASE
-    ROCM_LAUNCH_CHECK();
     hipLaunchKernelGGL((rmsNormBwdFold<T, ColAcc>), dim3(static_cast<unsigned>(ceilDiv(n2, 64))), dim3(256), 0, stream, static_cast<T*>(gW.data),
                        static_cast<T*>(gBias), partW, partB, numParts, n2);
     ROCM_LAUNCH_CHECK();

@@ -155,6 +155,119 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttMfma(T* __restrict__ out,
     }
 }
 
+// LDS-staged variant for D == 128.  The direct kernel above asks the memory pipeline for 16 different
+// cache rows per load instruction (64 bytes of each); this one loads the way the cache is laid out
+// and lets LDS do the re-shaping:
+//   * 16 consecutive lanes read one head row (256 contiguous bytes) of one token; a wave owns HW
+//     adjacent kv heads, so it reads HW*256 contiguous bytes per token and the waves of a work-group
+//     cover adjacent head ranges of the same tokens;
+//   * the 16 loads a lane issues per unit (TU = 64/HW tokens x HW heads) are all in flight before the
+//     first use; each [16 tokens x 128 dims] block then goes through a wave-private LDS tile
+//     (row pitch 272 bytes: conflict-free for both the 16-byte row writes and the 16-byte
+//     column-block reads) and comes back in the MFMA B-operand layout;
+//   * LDS operations of one wave execute in order, so the private tile needs no barrier.
+// Waves are mapped to (head slot, token phase): with few kv heads the spare waves take other units.
+constexpr int kStagePitch = 136;  // elements per staged row: 128 + 8
+
+template <typename T, int HW>
+__global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, DecodeArgs a, int TT,
+                                                              int HS, float scale) {
+    using Ops = MfmaOps<T>;
+    using Frag = typename Ops::Frag;
+    constexpr int D = 128;
+    constexpr int KSTEPS = D / 32;
+    constexpr int TU = 64 / HW;   // tokens per unit
+    constexpr int NJ = TU / 4;    // loads per head per lane in a unit (4 tokens per load instruction)
+    constexpr int NG = TU / 16;   // MFMA column groups per unit
+    __shared__ __attribute__((aligned(16))) T stage[kAttWaves][16 * kStagePitch];
+    __shared__ int sSlot[1024];   // slot index of every token of the tile (TT <= 1024)
+
+    const int i = blockIdx.y;
+    int64_t L = loadIndex(a.bSeqLen, i, a.len64);
+    if (L > a.maxInputLen) L = a.maxInputLen;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TT;
+    if (t0 >= L) return;
+    const int nTok = static_cast<int>((L - t0 < TT) ? L - t0 : TT);
+    const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
+    const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L) + t0;
+    for (int t = threadIdx.x; t < TT; t += kAttThreads) {
+        const int tc = t < nTok ? t : nTok - 1;  // tail tokens alias the last valid one; their results are not stored
+        int64_t slot = loadIndex(a.bLoc, locBase + tc, a.loc64);
+        slot = slot < 0 ? 0 : (slot >= a.numSlots ? a.numSlots - 1 : slot);
+        sSlot[t] = static_cast<int>(slot);
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane / 16;  // loads: token inside a quad; MFMA: k block (kq)
+    const int c = lane % 16;  // loads: 16-byte packet of the head row; MFMA: token column / query-head row (n)
+    const int TPH = kAttWaves / HS;
+    const int hs = wave % HS;
+    const int tph = wave / HS;
+    const int hk0 = (blockIdx.z * HS + hs) * HW;
+    if (hk0 >= a.Hkv) return;
+    const int64_t rowStride = static_cast<int64_t>(a.Hkv) * D;
+    T* myStage = stage[wave];
+
+    // A fragments of this wave's heads: row c is query head (hk0+u)*G + c, k slot (r, e) <-> dim 32*s + 8*r + e
+    Frag qa[HW][KSTEPS];
+#pragma unroll
+    for (int u = 0; u < HW; ++u) {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            const bool valid = c < a.G && hk0 + u < a.Hkv;
+            qa[u][s] = valid ? loadFrag<Frag>(q + (static_cast<int64_t>(i) * a.H + (hk0 + u) * a.G + c) * D + s * 32 + r * 8) : zeroFrag<Frag>();
+        }
+    }
+
+    const int numUnits = (nTok + TU - 1) / TU;
+    for (int unit = tph; unit < numUnits; unit += TPH) {
+        const int tu0 = unit * TU;
+        // every load of the unit is issued before the first use
+        u32x4 kv[NJ][HW];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int64_t rowOff = static_cast<int64_t>(sSlot[tu0 + 4 * j + r]) * rowStride;
+#pragma unroll
+            for (int u = 0; u < HW; ++u) {
+                const int hk = (hk0 + u < a.Hkv) ? hk0 + u : a.Hkv - 1;
+                kv[j][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k + rowOff + hk * D + c * 8));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < HW; ++u) {
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                // 16 tokens x 128 dims of head u: rows 4*jj + r of the private tile
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) *reinterpret_cast<u32x4*>(myStage + (4 * jj + r) * kStagePitch + c * 8) = kv[4 * g + jj][u];
+                __builtin_amdgcn_wave_barrier();  // keep the tile writes ahead of the reads in program order
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KSTEPS; ++s) {
+                    const Frag kb = loadFrag<Frag>(myStage + c * kStagePitch + s * 32 + r * 8);
+                    acc = Ops::mma(qa[u][s], kb, acc);
+                }
+                __builtin_amdgcn_wave_barrier();  // ... and the reads ahead of the next tile's writes
+                // C: this lane holds query heads 4*r + rr of token column c
+                const int t = tu0 + g * 16 + c;
+                const int64_t col = start + t0 + t;
+                if (t < nTok && hk0 + u < a.Hkv && col >= 0 && col < a.logitCols) {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int gh = 4 * r + rr;
+                        if (gh < a.G) {
+                            const T dot = static_cast<T>(acc[rr]);
+                            out[static_cast<int64_t>((hk0 + u) * a.G + gh) * a.logitCols + col] = static_cast<T>(static_cast<float>(dot) * scale);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
 // Any dtype / head size / grouping: one thread per (token, query head) pair of a tile.
 template <typename T, typename AccT>
 __global__ __launch_bounds__(kAttThreads) void tokenAttGeneric(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, DecodeArgs a, int TT,
@@ -204,6 +317,34 @@ diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void
     return diopiSuccess;
 }
 
+template <typename T>
+diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a, float scale) {
+    // heads per wave, head slots per work-group (waves beyond the head slots take other token units)
+    const int HW = a.Hkv >= 16 ? 4 : (a.Hkv >= 8 ? 2 : 1);
+    const int slots = static_cast<int>(ceilDiv(a.Hkv, HW));
+    const int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
+    // tokens per work-group: about half a MiB of K per group
+    int TT = static_cast<int>((512 * 1024) / (static_cast<int64_t>(HS) * HW * 128 * sizeof(T)));
+    TT = envInt("DIOPI_ROCM_TOKATT_TT", TT);
+    TT = TT / 64 * 64;
+    if (TT < 64) TT = 64;
+    if (TT > 1024) TT = 1024;
+    const dim3 grid(static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)));
+#define ROCM_STAGED_CASE(HWC)                                                                                                                         \
+    hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),                  \
+                       static_cast<const T*>(k), a, TT, HS, scale)
+    if (HW == 4) {
+        ROCM_STAGED_CASE(4);
+    } else if (HW == 2) {
+        ROCM_STAGED_CASE(2);
+    } else {
+        ROCM_STAGED_CASE(1);
+    }
+#undef ROCM_STAGED_CASE
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
 template <typename T, typename AccT>
 diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a) {
     const int TT = 64;
@@ -242,10 +383,13 @@ extern "C" diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, d
                       envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
     // the element type's matmul rounds the fp32 dot to T, then the division by sqrt(D) rounds again
     const float scale = 1.0f / static_cast<float>(std::sqrt(static_cast<double>(D)));
+    const bool staged = fast && D == 128 && envInt("DIOPI_ROCM_TOKATT_DIRECT", 0) == 0;
     switch (vQ.dtype) {
         case diopi_dtype_float16:
+            if (staged) return launchStaged<half_t>(stream, vOut.data, vQ.data, vK.data, a, scale);
             return fast ? launchMfma<half_t>(stream, vOut.data, vQ.data, vK.data, a, scale) : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, a);
         case diopi_dtype_bfloat16:
+            if (staged) return launchStaged<bf16_t>(stream, vOut.data, vQ.data, vK.data, a, scale);
             return fast ? launchMfma<bf16_t>(stream, vOut.data, vQ.data, vK.data, a, scale) : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, a);
         case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, a);
         case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, a);
