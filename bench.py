@@ -323,9 +323,9 @@ def main():
         line["config"]["total_cached_tokens"] = head["total"]
         # dominant kernel of the step: the slower of the two attention halves
         if head["ms_att"] >= head["ms_red"]:
-            kname, kms, kbytes = "tokenAttMfma (diopiTokenAttentionInference)", head["ms_att"], head["b_att"]
+            kname, kms, kbytes = "tokenAttStaged (diopiTokenAttentionInference)", head["ms_att"], head["b_att"]
         else:
-            kname, kms, kbytes = "softmaxReduceVSplit+Merge (diopiTokenSoftmaxReduceVInference)", head["ms_red"], head["b_red"]
+            kname, kms, kbytes = "softmaxReduceVWave+Merge (diopiTokenSoftmaxReduceVInference)", head["ms_red"], head["b_red"]
         ach = kbytes / (kms * 1e-3) / 1e9
         line["roofline"] = {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                             "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}

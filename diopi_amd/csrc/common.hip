@@ -11,17 +11,17 @@
 namespace rocm {
 
 // ---- last error ------------------------------------------------------------
-// One process-wide message behind a mutex, as in impl/torch/functions/error.cpp:13-29 of the
-// reference: the text returned by diopiGetLastErrorString() is "<device error>; other error: <message>".
+// The text returned by diopiGetLastErrorString() is "<device error>; other error: <message>", as in
+// impl/torch/functions/error.cpp:13-29 of the reference.  The reference keeps one process-wide buffer behind a
+// mutex, which still hands the caller a pointer another thread may be rewriting; here every host thread has its
+// own message, so the pointer stays valid and describes the calling thread's last failure.
 namespace {
-char gLastErrorText[4096] = {0};
-char gLastErrorOther[2048] = {0};
-char gLastHipError[256] = "no error";
-std::mutex gLastErrorMutex;
+thread_local char gLastErrorText[4096] = {0};
+thread_local char gLastErrorOther[2048] = {0};
+thread_local char gLastHipError[256] = "no error";
 }  // namespace
 
 void setLastError(const char* fmt, ...) {
-    std::lock_guard<std::mutex> lock(gLastErrorMutex);
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(gLastErrorOther, sizeof(gLastErrorOther), fmt, ap);
@@ -29,7 +29,6 @@ void setLastError(const char* fmt, ...) {
 }
 
 void setLastErrorAt(const char* file, int line, const char* fmt, ...) {
-    std::lock_guard<std::mutex> lock(gLastErrorMutex);
     const char* base = std::strrchr(file, '/');
     int n = snprintf(gLastErrorOther, sizeof(gLastErrorOther), "%s:%d: ", base ? base + 1 : file, line);
     if (n < 0 || n >= static_cast<int>(sizeof(gLastErrorOther))) return;
@@ -40,12 +39,10 @@ void setLastErrorAt(const char* file, int line, const char* fmt, ...) {
 }
 
 void noteHipError(hipError_t err) {
-    std::lock_guard<std::mutex> lock(gLastErrorMutex);
     snprintf(gLastHipError, sizeof(gLastHipError), "%s", hipGetErrorString(err));
 }
 
 static const char* lastErrorString() {
-    std::lock_guard<std::mutex> lock(gLastErrorMutex);
     snprintf(gLastErrorText, sizeof(gLastErrorText), "hip error: %s; other error: %s", gLastHipError, gLastErrorOther);
     return gLastErrorText;
 }

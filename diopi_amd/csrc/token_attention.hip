@@ -84,10 +84,13 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttMfma(T* __restrict__ out,
     using Ops = MfmaOps<T>;
     using Frag = typename Ops::Frag;
     constexpr int kGroups = TT / kTokGroup;
-    const int i = blockIdx.y;
+    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
+    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
+    // sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
     if (t0 >= L) return;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int lane = threadIdx.x % kWave;
@@ -182,10 +185,13 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     __shared__ __attribute__((aligned(16))) T stage[kAttWaves][16 * kStagePitch];
     __shared__ int sSlot[1024];   // slot index of every token of the tile (TT <= 1024)
 
-    const int i = blockIdx.y;
+    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
+    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
+    // sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
     if (t0 >= L) return;
     const int nTok = static_cast<int>((L - t0 < TT) ? L - t0 : TT);
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
@@ -272,10 +278,13 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
 template <typename T, typename AccT>
 __global__ __launch_bounds__(kAttThreads) void tokenAttGeneric(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, DecodeArgs a, int TT,
                                                                AccT scale) {
-    const int i = blockIdx.y;
+    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
+    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
+    // sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
     if (t0 >= L) return;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L);
@@ -305,7 +314,7 @@ diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void
     // kv heads per work-group: about 256 KiB of K per group, at least one head per wave
     int HB = a.Hkv < 8 ? a.Hkv : 8;
     HB = envInt("DIOPI_ROCM_TOKATT_HB", HB);
-    const dim3 grid(static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.Hkv, HB)));
+    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(ceilDiv(a.Hkv, HB)));
     if (a.D == 128) {
         hipLaunchKernelGGL((tokenAttMfma<T, 4, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
                            static_cast<const T*>(k), a, HB, scale);
@@ -329,7 +338,7 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     TT = TT / 64 * 64;
     if (TT < 64) TT = 64;
     if (TT > 1024) TT = 1024;
-    const dim3 grid(static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)));
+    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)));
 #define ROCM_STAGED_CASE(HWC)                                                                                                                         \
     hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),                  \
                        static_cast<const T*>(k), a, TT, HS, scale)
@@ -348,7 +357,7 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
 template <typename T, typename AccT>
 diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a) {
     const int TT = 64;
-    const dim3 grid(static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch));
+    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
     const AccT scale = static_cast<AccT>(1.0 / std::sqrt(static_cast<double>(a.D)));
     hipLaunchKernelGGL((tokenAttGeneric<T, AccT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
                        static_cast<const T*>(k), a, TT, scale);

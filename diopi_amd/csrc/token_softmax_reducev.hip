@@ -8,20 +8,12 @@
 //   out[i, h, :] = sum_t P[t] * v[slots[t], h / G, :]                         (fp32 accumulate)
 // other_kv_index is ignored, as in the reference.
 //
-// Kernel shape (16-bit types, D == 128): a split-K ("flash decoding") pass followed by a small
-// merge.  A work-group owns (token range, sequence, group of HB kv heads).  It walks its range in
-// sub-tiles of 128 tokens:
-//   1. each wave takes query heads of the group in turn, reads the sub-tile's logits as one
-//      coalesced row segment, updates the running maximum / denominator of that head and leaves
-//      the un-normalised probabilities exp(x - max) in LDS together with the rescale factor;
-//   2. 16 lanes own one V row segment (one kv head of one token, 256 bytes, one 16-byte load per
-//      lane); the 16 such lane groups of the work-group cover HB heads x 16/HB tokens per step.
-//      Each lane multiplies its 8 V elements by the probabilities of the G query heads sharing
-//      that kv head and accumulates in fp32 registers.  V bytes are read exactly once.
-// At the end the lane groups that worked on the same head are summed through LDS and the range's
-// (max, denominator, accumulator) triple is written to context-owned scratch; a merge kernel
-// combines the ranges of a sequence.  A sequence that fits one range is finished in place and
-// skips the scratch round trip.  Nothing on the host depends on the sequence lengths.
+// Kernel shape (16-bit types, D == 128, G <= 16): a split-K ("flash decoding") pass on the matrix cores followed
+// by a small merge.  A wave owns (kv head, token range, sequence); it never synchronises with other waves.  The
+// range's (max, denominator, accumulator) triple goes to context-owned scratch and a merge kernel combines the
+// ranges of a sequence; a sequence that fits one range is finished in place and skips the scratch round trip.
+// V bytes are read exactly once.  Nothing on the host depends on the sequence lengths.
+// Everything else (fp32 / fp64, other head sizes, G > 16) takes a shape-agnostic kernel.
 #include <cmath>
 
 #include "common.hpp"
@@ -34,29 +26,27 @@ namespace {
 constexpr int kRvThreads = 256;
 constexpr int kRvWaves = kRvThreads / kWave;
 constexpr int kSub = 128;          // tokens per sub-tile
-constexpr int kLaneGroups = 16;    // 16-lane groups per work-group
-constexpr int kMaxHeadsQ = 64;     // query heads per work-group (HB * G) the LDS tile is sized for
 constexpr int kD = 128;
 
-// c + a.lo*b.lo + a.hi*b.hi on packed 16-bit pairs, accumulated in fp32 (v_dot2_f32_f16 / v_dot2_f32_bf16).
-// The last argument only selects the element type.
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c, half_t*) {
-    union {
-        uint32_t u;
-        f16x2 v;
-    } ua, ub;
-    ua.u = a;
-    ub.u = b;
-    return __builtin_amdgcn_fdot2(ua.v, ub.v, c, false);
+// Reductions over the 16 lanes of a DPP row (quad permutes, then half-row and full-row mirrors); every lane of the
+// row ends with the result.  Four VALU moves instead of four trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dppMove(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c, bf16_t*) {
-    union {
-        uint32_t u;
-        bf16x2 v;
-    } ua, ub;
-    ua.u = a;
-    ub.u = b;
-    return __builtin_amdgcn_fdot2_f32_bf16(ua.v, ub.v, c, false);
+__device__ __forceinline__ float rowMax16(float v) {
+    v = fmaxf(v, dppMove<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dppMove<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dppMove<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dppMove<0x140>(v));  // row_mirror
+    return v;
+}
+__device__ __forceinline__ float rowSum16(float v) {
+    v += dppMove<0xB1>(v);
+    v += dppMove<0x4E>(v);
+    v += dppMove<0x141>(v);
+    v += dppMove<0x140>(v);
+    return v;
 }
 
 struct SplitArgs {
@@ -64,380 +54,237 @@ struct SplitArgs {
     float* partMl;   // [batch, splits, H, 2]  (running max, denominator)
     int splits;      // ranges per sequence the scratch is sized for
     int TT;          // tokens per range (multiple of kSub)
-    int HB;          // kv heads per work-group: 1, 2, 4, 8 or 16
 };
 
-template <typename T, int G>
-__global__ __launch_bounds__(kRvThreads) void softmaxReduceVSplit(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
-                                                                  SplitArgs sp) {
-    // un-normalised probabilities of the sub-tile; after the sweep the same storage holds the
-    // [query head][dim] sums over the token phases
-    __shared__ float sP[kMaxHeadsQ][kSub];
-    __shared__ float sAlpha[kMaxHeadsQ];        // rescale factor of the accumulators for this sub-tile
-    __shared__ float sM[kMaxHeadsQ];            // running maximum per query head
-    __shared__ float sL[kMaxHeadsQ];            // running denominator per query head
-    __shared__ int64_t sSlot[kSub];             // element offset of each token's cache row
+// Matrix-core kernel (16-bit types, D == 128, any G <= 16): per kv head the weighted sum is the small product
+//   out[g, d] += P[g, t] . V[t, d]      on v_mfma_f32_16x16x32 (16 query heads x 16 dims x 32 tokens),
+// so the vector-ALU work per V byte does not grow with G.
+// A wave owns (kv head, token range, sequence), i.e. the G query heads of its kv head, and walks the range in
+// sub-tiles of 128 tokens without ever meeting another wave at a barrier:
+//   * logits of the sub-tile: per query head two coalesced loads (lane = token), prefetched one sub-tile ahead;
+//     running maximum / denominator per head are wave-uniform values (DPP row reduction + four lane reads);
+//     the probabilities go to a wave-private LDS tile [G][128 + 8] in the element type;
+//   * cache slots of the next sub-tile are fetched one sub-tile ahead and parked in wave-private LDS;
+//   * V rows: the four 16-lane groups read the rows of 8 tokens each (one 16-byte load per lane and row, 8 rows in
+//     flight per lane).  MFMA wants the contraction index (tokens) inside a lane's registers while a row is contiguous
+//     along d; since 16-bit operands travel as pairs, interleaving the registers of rows (t, t+1) with two byte
+//     permutes turns the 8 loaded rows into the B operands of the lane's 8 dims: 4 permutes per row, no LDS, no
+//     second pass over the data.  The first rows of the next sub-tile are requested before its softmax work starts,
+//     so the wave always has rows in flight;
+//   * the A operand (8 consecutive tokens of query head l % 16) is one 16-byte read of the probability tile;
+//   * C holds out[4 * (l / 16) + r][8 * (l % 16) + e] in acc[e][r]: a lane ends up with 8 consecutive dims of up to
+//     four query heads, which are stored directly; accumulator rows are rescaled only when some head's maximum
+//     moved (a wave-uniform test).
+constexpr int kTilePitch = kSub + 8;  // elements per probability row; 272 bytes
 
-    const int i = blockIdx.y;
-    int64_t L = loadIndex(a.bSeqLen, i, a.len64);
-    if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * sp.TT;
-    if (t0 >= L) return;
-    const int64_t tEnd = (t0 + sp.TT < L) ? t0 + sp.TT : L;
-    const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
-    const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L);
-    const int tid = threadIdx.x;
-    const int lane = tid % kWave;
-    const int wave = tid / kWave;
-    const int HB = sp.HB;
-    const int hkBegin = blockIdx.z * HB;
-    const int headsQ = HB * G;  // query heads handled here (some may lie beyond H when Hkv % HB != 0)
-
-    // lane group -> (kv head inside the group, token phase)
-    const int lg = tid / 16;
-    const int c = tid % 16;  // 16-byte packet of the 256-byte row segment
-    const int hl = lg % HB;  // local kv head
-    const int tp = lg / HB;  // token phase
-    const int TP = kLaneGroups / HB;
-    const int hk = hkBegin + hl;
-    const bool headValid = hk < a.Hkv;
-    const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
-
-    float acc[G][8];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
-    }
-    for (int h = tid; h < headsQ; h += kRvThreads) {
-        sM[h] = -INFINITY;
-        sL[h] = 0.f;
-    }
-    __syncthreads();
-
-    for (int64_t ts = t0; ts < tEnd; ts += kSub) {
-        const int nTok = static_cast<int>((tEnd - ts < kSub) ? tEnd - ts : kSub);
-        // ---- phase 1: slots and probabilities of the sub-tile ----
-        for (int t = tid; t < kSub; t += kRvThreads) {
-            // tokens past the end alias the last valid one (their probability is zero)
-            int64_t slot = loadIndex(a.bLoc, locBase + ts + (t < nTok ? t : nTok - 1), a.loc64);
-            slot = slot < 0 ? 0 : (slot >= a.numSlots ? a.numSlots - 1 : slot);
-            sSlot[t] = slot * rowStride;
-        }
-        for (int h = wave; h < headsQ; h += kRvWaves) {
-            const int qh = hkBegin * G + h;
-            float x[kSub / kWave];
-            float mloc = -INFINITY;
-#pragma unroll
-            for (int j = 0; j < kSub / kWave; ++j) {
-                const int t = j * kWave + lane;
-                const int64_t col = start + ts + t;
-                x[j] = -INFINITY;
-                if (t < nTok && qh < a.H && col >= 0 && col < a.logitCols) x[j] = static_cast<float>(logits[static_cast<int64_t>(qh) * a.logitCols + col]);
-                mloc = fmaxf(mloc, x[j]);
-            }
-            mloc = waveMax(mloc);
-            const float mOld = sM[h];
-            const float mNew = fmaxf(mOld, mloc);
-            float lsum = 0.f;
-#pragma unroll
-            for (int j = 0; j < kSub / kWave; ++j) {
-                const int t = j * kWave + lane;
-                // a row of -inf logits keeps p = 0 instead of exp(nan)
-                const float p = (x[j] == -INFINITY) ? 0.f : __expf(x[j] - mNew);
-                if constexpr (G == 1) {
-                    sP[h][t] = p;
-                } else {
-                    // grouped heads: probabilities rounded to the element type and stored as token pairs,
-                    // [token pair][query head] -> one dword per (pair, head), the operand layout of the dot2 path
-                    reinterpret_cast<T*>(&sP[0][0])[((t >> 1) * kMaxHeadsQ + h) * 2 + (t & 1)] = static_cast<T>(p);
-                }
-                lsum += p;
-            }
-            lsum = waveSum(lsum);
-            if (lane == 0) {
-                const float alpha = (mOld == -INFINITY) ? 0.f : __expf(mOld - mNew);
-                sAlpha[h] = alpha;
-                sM[h] = mNew;
-                sL[h] = sL[h] * alpha + lsum;
-            }
-        }
-        __syncthreads();
-        // ---- phase 2: accumulate V rows ----
-        if (headValid) {
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                const float alpha = sAlpha[hl * G + g];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[g][e] *= alpha;
-            }
-            const T* vHead = v + hk * kD + c * 8;
-            constexpr int U = 8;  // rows in flight per lane
-            if constexpr (G > 1) {
-                // Two tokens at a time: the rows of tokens (t, t+1) are interleaved element-wise with byte permutes
-                // and multiplied against the packed probability pairs with v_dot2 (fp32 accumulate): half the VALU
-                // work of convert + fma per element, which is what bounds this kernel once G query heads share a row.
-                const uint32_t* sPairs = reinterpret_cast<const uint32_t*>(&sP[0][0]);
-                const int nPairs = (nTok + 1) / 2;
-                constexpr int UP = U / 2;
-                for (int pb = tp; pb < nPairs; pb += TP * UP) {
-                    u32x4 v0[UP], v1[UP];
-#pragma unroll
-                    for (int u = 0; u < UP; ++u) {
-                        const int pr = pb + u * TP;
-                        if (pr < nPairs) {
-                            v0[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + sSlot[2 * pr]));
-                            v1[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + sSlot[2 * pr + 1]));
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < UP; ++u) {
-                        const int pr = pb + u * TP;
-                        if (pr < nPairs) {
-                            uint32_t pp[G];
-#pragma unroll
-                            for (int g = 0; g < G; ++g) pp[g] = sPairs[pr * kMaxHeadsQ + hl * G + g];
-#pragma unroll
-                            for (int kk = 0; kk < 4; ++kk) {
-                                // (row t elem 2kk, row t+1 elem 2kk) and (row t elem 2kk+1, row t+1 elem 2kk+1)
-                                const uint32_t lo = __builtin_amdgcn_perm(v1[u][kk], v0[u][kk], 0x05040100u);
-                                const uint32_t hi = __builtin_amdgcn_perm(v1[u][kk], v0[u][kk], 0x07060302u);
-#pragma unroll
-                                for (int g = 0; g < G; ++g) {
-                                    acc[g][2 * kk] = dot2(lo, pp[g], acc[g][2 * kk], static_cast<T*>(nullptr));
-                                    acc[g][2 * kk + 1] = dot2(hi, pp[g], acc[g][2 * kk + 1], static_cast<T*>(nullptr));
-                                }
-                            }
-                        }
-                    }
-                }
-            } else
-            for (int tb = tp; tb < nTok; tb += TP * U) {
-                Pack16<T> vv[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int t = tb + u * TP;
-                    if (t < nTok) vv[u] = loadPackStream(vHead + sSlot[t]);
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int t = tb + u * TP;
-                    if (t < nTok) {
-                        float vf[8];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) vf[e] = static_cast<float>(vv[u].e[e]);
-#pragma unroll
-                        for (int g = 0; g < G; ++g) {
-                            const float p = sP[hl * G + g][t];
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) acc[g][e] += p * vf[e];
-                        }
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- fold the token phases (kSub == kD, so sP doubles as a [query head][dim] buffer) ----
-    static_assert(kSub == kD, "the probability tile is reused as the fold buffer");
-    for (int p = 0; p < TP; ++p) {
-        if (tp == p && headValid) {
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float* dst = &sP[hl * G + g][c * 8 + e];
-                    *dst = (p == 0) ? acc[g][e] : *dst + acc[g][e];
-                }
-            }
-        }
-        __syncthreads();
-    }
-    const bool single = L <= sp.TT;  // the whole sequence lives in this range
-    const int64_t split = blockIdx.x;
-    for (int idx = tid; idx < headsQ * kD; idx += kRvThreads) {
-        const int h = idx / kD;   // local query head = hl * G + g
-        const int d = idx % kD;
-        const int hlq = h / G, g = h % G;
-        const int qh = hkBegin * G + h;
-        if (hkBegin + hlq >= a.Hkv || qh >= a.H) continue;
-        (void)g;
-        const float s = sP[h][d];
-        if (single) {
-            out[(static_cast<int64_t>(i) * a.H + qh) * kD + d] = static_cast<T>(s / sL[h]);
-        } else {
-            sp.partAcc[((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * kD + d] = s;
-        }
-    }
-    if (!single) {
-        for (int h = tid; h < headsQ; h += kRvThreads) {
-            const int qh = hkBegin * G + h;
-            if (hkBegin + h / G >= a.Hkv || qh >= a.H) continue;
-            float* ml = sp.partMl + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * 2;
-            ml[0] = sM[h];
-            ml[1] = sL[h];
-        }
-    }
+// LDS that only one wave touches needs no barrier (the LDS executes a wave's operations in order), but the compiler
+// must not move accesses of different types across the hand-over points.
+__device__ __forceinline__ void waveLdsFence() {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+}
+__device__ __forceinline__ float laneValue(float v, int l) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float waveMaxUniform(float v) {
+    v = rowMax16(v);
+    return fmaxf(fmaxf(laneValue(v, 0), laneValue(v, 16)), fmaxf(laneValue(v, 32), laneValue(v, 48)));
+}
+__device__ __forceinline__ float waveSumUniform(float v) {
+    v = rowSum16(v);
+    return (laneValue(v, 0) + laneValue(v, 16)) + (laneValue(v, 32) + laneValue(v, 48));
 }
 
-// Grouped-head variant (G query heads share one kv head, 2 <= G <= 16): the weighted sum becomes a small matrix
-// product per kv head,  out^T[d, g] += V^T[d, t] . P^T[t, g],  on v_mfma_f32_16x16x32 (16 dims x 16 heads x 32 tokens),
-// so the per-byte VALU cost no longer grows with G.
-//   * a wave owns one kv head of one token range; it reads each V row segment (256 bytes) with 16 adjacent lanes, eight
-//     16-byte loads per lane in flight, and parks the [32 tokens x 128 dims] block in a wave-private LDS tile;
-//   * the A operand (8 tokens of one dim per lane) is gathered from the tile with 16-bit reads; the tile columns are
-//     XOR-swizzled by (token / 8) in units of 16 dims so that the four k blocks of a wave hit disjoint LDS banks;
-//   * the B operand (8 consecutive tokens of one query head per lane) is read straight from the logits tensor, which is
-//     head-major, and exponentiated in registers: the softmax statistics of head g live in the lanes with l % 16 == g
-//     and the running maximum / denominator / rescale never leave registers (two cross-lane exchanges per 32 tokens);
-//   * every wave writes its own (max, denominator, accumulator) partial; softmaxReduceVMerge combines them.
-constexpr int kVTileTokens = 32;
-constexpr int kVTilePitch = kD + 8;  // elements; 272 bytes
-
-template <typename T>
-__global__ __launch_bounds__(kRvThreads) void softmaxReduceVMfma(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
-                                                                 SplitArgs sp, int HS) {
+template <typename T, int GC>
+__global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
+                                                                    SplitArgs sp) {
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
-    __shared__ __attribute__((aligned(16))) T tile[kRvWaves][kVTileTokens * kVTilePitch];
-    const int i = blockIdx.y;
+    __shared__ __attribute__((aligned(16))) T sP[kRvWaves][GC * kTilePitch];
+    __shared__ __attribute__((aligned(16))) int32_t sSlotW[kRvWaves][kSub];
+    __shared__ __attribute__((aligned(16))) float sStat[kRvWaves][16];
+
+    // x runs over sequences, y over token ranges, rotated so that consecutive work-groups (dealt round-robin to the 8
+    // XCDs) mix ranges of different sequences: with ragged lengths no XCD is left with only the sparse late ranges
+    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int lane = threadIdx.x % kWave;
-    const int wave = threadIdx.x / kWave;
-    const int TPH = kRvWaves / HS;      // token ranges handled by this work-group
-    const int hs = wave % HS;
-    const int tph = wave / HS;
-    const int hk = blockIdx.z * HS + hs;
-    const int64_t split = static_cast<int64_t>(blockIdx.x) * TPH + tph;
-    const int64_t t0 = split * sp.TT;
-    if (hk >= a.Hkv || t0 >= L) return;  // no work-group barrier below: waves are independent
+    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * sp.TT;
+    if (t0 >= L) return;
     const int64_t tEnd = (t0 + sp.TT < L) ? t0 + sp.TT : L;
+    const int nTokR = static_cast<int>(tEnd - t0);
+    const int nSub = (nTokR + kSub - 1) / kSub;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
-    const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L);
-    const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
-    const int n = lane % 16;   // A: dim inside a 16-dim block; B and C: query head inside the group
-    const int kq = lane / 16;  // k block: tokens 8*kq .. 8*kq+7 of the tile; loads: token inside a quad
+    const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L) + t0;
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int q = lane / 16;  // 16-lane group: tokens 8q .. 8q+7 of every 32-token step
+    const int c = lane % 16;  // 16-byte packet of the row segment; also the query head of the A operand
     const int G = a.G;
-    const bool headOk = n < G;
-    const int qh = hk * G + n;
-    const T* logitRow = logits + static_cast<int64_t>(headOk ? qh : hk * G) * a.logitCols;
-    T* myTile = tile[wave];
-    const T* vHead = v + hk * kD + n * 8;  // loads: lane n covers packet n of the 256-byte row segment
+    const int hk = blockIdx.z * kRvWaves + wave;
+    if (hk >= a.Hkv) return;
+    const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
+    T* tile = &sP[wave][0];
+    int32_t* slotW = &sSlotW[wave][0];
+    float* statW = &sStat[wave][0];
+    const T* vHead = v + hk * kD + c * 8;
+    const int64_t colBase = start + t0;
+    const T* xBase = logits + static_cast<int64_t>(hk) * G * a.logitCols + colBase;
 
-    f32x4 acc[kD / 16];
+    // logits of sub-tile `sub`: xr[g][k] = logit of query head g, token 64k + lane (-inf outside the sequence)
+    float xr[GC][2];
+    auto loadLogits = [&](int sub) {
 #pragma unroll
-    for (int db = 0; db < kD / 16; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float mRun = -INFINITY, lRun = 0.f;
-
-    // Software pipeline, two tiles deep: slot indices are fetched two tiles ahead, V rows and logits one tile ahead,
-    // so that the dependent chain slot -> row address -> row never stalls the tile being multiplied.
-    constexpr int NJ = kVTileTokens / 4;
-    int64_t rowOff[NJ];
-    auto fetchSlots = [&](int64_t ts) {
+        for (int g = 0; g < GC; ++g) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            int64_t t = ts + 4 * j + kq;
-            if (t > tEnd - 1) t = tEnd - 1;  // tail tokens alias the last valid one; their probability is zero
+            for (int k = 0; k < 2; ++k) {
+                const int t = sub * kSub + 64 * k + lane;
+                const int64_t col = colBase + t;
+                xr[g][k] = -INFINITY;
+                if (g < G && t < nTokR && col >= 0 && col < a.logitCols) xr[g][k] = static_cast<float>(xBase[static_cast<int64_t>(g) * a.logitCols + t]);
+            }
+        }
+    };
+    int32_t slotNext[2];
+    auto loadSlots = [&](int sub) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            int t = sub * kSub + 64 * k + lane;
+            t = t < nTokR ? t : nTokR - 1;  // tokens past the end alias the last valid one (their probability is zero)
             int64_t slot = loadIndex(a.bLoc, locBase + t, a.loc64);
             slot = slot < 0 ? 0 : (slot >= a.numSlots ? a.numSlots - 1 : slot);
-            rowOff[j] = slot * rowStride;
+            slotNext[k] = static_cast<int32_t>(slot);
         }
     };
-    auto fetchRows = [&](u32x4* dst) {
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) dst[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + rowOff[j]));
+    auto storeSlots = [&]() {
+        waveLdsFence();
+        slotW[lane] = slotNext[0];
+        slotW[64 + lane] = slotNext[1];
+        waveLdsFence();
     };
-    auto fetchLogits = [&](int64_t ts, float* dst) {
+    u32x4 rowsV[8];
+    auto issueV = [&](int step) {
+        int32_t sidx[8];
+        *reinterpret_cast<u32x4*>(&sidx[0]) = *reinterpret_cast<const u32x4*>(slotW + 32 * step + 8 * q);
+        *reinterpret_cast<u32x4*>(&sidx[4]) = *reinterpret_cast<const u32x4*>(slotW + 32 * step + 8 * q + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int64_t t = ts + 8 * kq + e;
-            const int64_t col = start + t;
-            dst[e] = -INFINITY;
-            if (headOk && t < tEnd && col >= 0 && col < a.logitCols) dst[e] = static_cast<float>(logitRow[col]);
-        }
+        for (int r = 0; r < 8; ++r) rowsV[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(sidx[r]) * rowStride));
     };
-    u32x4 vv[NJ], vn[NJ];
-    float x[8], xn[8];
-    fetchSlots(t0);
-    fetchRows(vv);
-    fetchLogits(t0, x);
-    if (t0 + kVTileTokens < tEnd) fetchSlots(t0 + kVTileTokens);
 
-    for (int64_t ts = t0; ts < tEnd; ts += kVTileTokens) {
-        if (ts + kVTileTokens < tEnd) {
-            fetchRows(vn);
-            fetchLogits(ts + kVTileTokens, xn);
-            if (ts + 2 * kVTileTokens < tEnd) fetchSlots(ts + 2 * kVTileTokens);
-        }
-        float umax = -INFINITY;
+    loadSlots(0);
+    storeSlots();
+    issueV(0);
+    loadLogits(0);
+
+    f32x4 acc[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) umax = fmaxf(umax, x[e]);
-        umax = fmaxf(umax, __shfl_xor(umax, 16, kWave));
-        umax = fmaxf(umax, __shfl_xor(umax, 32, kWave));
-        const float mNew = fmaxf(mRun, umax);
-        const float alpha = (mRun == -INFINITY) ? 0.f : __expf(mRun - mNew);
-        Frag pf;
-        float psum = 0.f;
+    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mRun[GC], lRun[GC];  // wave-uniform
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float p = (x[e] == -INFINITY) ? 0.f : __expf(x[e] - mNew);
-            psum += p;
-            pf[e] = static_cast<T>(p);
-        }
-        lRun = lRun * alpha + psum;  // this lane's share; the four k blocks are added at the end
-        mRun = mNew;
-#pragma unroll
-        for (int db = 0; db < kD / 16; ++db) {
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) acc[db][rr] *= alpha;
-        }
-        // ---- park the V block: row = token, 16-byte packet index XOR-ed with 2 * (token / 8) ----
-#pragma unroll
-        for (int j = 0; j < kVTileTokens / 4; ++j) {
-            const int t = 4 * j + kq;
-            *reinterpret_cast<u32x4*>(myTile + t * kVTilePitch + ((n ^ (((t >> 3) & 3) << 1)) * 8)) = vv[j];
-        }
-        __builtin_amdgcn_wave_barrier();
-        // ---- out^T[16*db + m, g] += sum_t V[t, 16*db + m] * P[t, g] ----
-#pragma unroll
-        for (int db = 0; db < kD / 16; ++db) {
-            Frag vf;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) vf[e] = myTile[(8 * kq + e) * kVTilePitch + 16 * (db ^ kq) + n];
-            acc[db] = Ops::mma(vf, pf, acc[db]);
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) vv[j] = vn[j];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = xn[e];
+    for (int g = 0; g < GC; ++g) {
+        mRun[g] = -INFINITY;
+        lRun[g] = 0.f;
     }
 
-    // ---- this wave's partial: lane (n = head, kq) holds dims 16*db + 4*kq + rr ----
-    lRun += __shfl_xor(lRun, 16, kWave);
-    lRun += __shfl_xor(lRun, 32, kWave);
-    if (!headOk) return;
-    const bool single = L <= sp.TT;
-    if (single) {
-        const float inv = 1.0f / lRun;
-        T* o = out + (static_cast<int64_t>(i) * a.H + qh) * kD;
+    for (int sub = 0; sub < nSub; ++sub) {
+        const int nTok = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
+        const int nSteps = (nTok + 31) / 32;
+        // ---- softmax of the sub-tile ----
+        waveLdsFence();
+        bool moved = false;
 #pragma unroll
-        for (int db = 0; db < kD / 16; ++db) {
-            T pk[4];
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) pk[rr] = static_cast<T>(acc[db][rr] * inv);
-            *reinterpret_cast<u32x2*>(o + 16 * db + 4 * kq) = *reinterpret_cast<const u32x2*>(pk);
+        for (int g = 0; g < GC; ++g) {
+            if (g < G) {
+                const float mNew = fmaxf(mRun[g], waveMaxUniform(fmaxf(xr[g][0], xr[g][1])));
+                const float mUse = (mNew == -INFINITY) ? 0.f : mNew;  // a head whose logits are all -inf keeps p = 0
+                const float p0 = __expf(xr[g][0] - mUse);
+                const float p1 = __expf(xr[g][1] - mUse);
+                const float alpha = (mRun[g] == -INFINITY) ? 0.f : __expf(mRun[g] - mNew);
+                moved = moved || (mNew != mRun[g]);
+                lRun[g] = lRun[g] * alpha + waveSumUniform(p0 + p1);
+                mRun[g] = mNew;
+                tile[g * kTilePitch + lane] = static_cast<T>(p0);
+                tile[g * kTilePitch + 64 + lane] = static_cast<T>(p1);
+                if (lane == 0) statW[g] = alpha;
+            }
         }
-    } else {
-        float* pa = sp.partAcc + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * kD;
+        if (sub + 1 < nSub) {
+            loadLogits(sub + 1);
+            loadSlots(sub + 1);
+        }
+        waveLdsFence();
+        if (moved) {
+            const f32x4 al = *reinterpret_cast<const f32x4*>(statW + 4 * q);
 #pragma unroll
-        for (int db = 0; db < kD / 16; ++db) *reinterpret_cast<f32x4*>(pa + 16 * db + 4 * kq) = acc[db];
-        if (kq == 0) {
-            float* ml = sp.partMl + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * 2;
-            ml[0] = mRun;
-            ml[1] = lRun;
+            for (int e = 0; e < 8; ++e) acc[e] *= al;
+        }
+        // ---- P . V on the matrix cores ----
+        const T* pRow = tile + (c < G ? c : 0) * kTilePitch + 8 * q;
+        for (int s = 0; s < nSteps; ++s) {
+            union {
+                u32x4 u;
+                Frag f;
+            } pa;
+            pa.u = *reinterpret_cast<const u32x4*>(pRow + 32 * s);
+            if (c >= G) pa.u = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                union {
+                    u32x4 u;
+                    Frag f;
+                } lo, hi;
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    // dims 2j and 2j+1 of this lane's packet, tokens (2pr, 2pr+1) of the lane group
+                    lo.u[pr] = __builtin_amdgcn_perm(rowsV[2 * pr + 1][j], rowsV[2 * pr][j], 0x05040100u);
+                    hi.u[pr] = __builtin_amdgcn_perm(rowsV[2 * pr + 1][j], rowsV[2 * pr][j], 0x07060302u);
+                }
+                acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
+                acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
+            }
+            // the row registers are free again: request the next rows (of this sub-tile or the first of the next one)
+            if (s + 1 < nSteps) {
+                issueV(s + 1);
+            } else if (sub + 1 < nSub) {
+                storeSlots();
+                issueV(0);
+            }
+        }
+    }
+
+    // ---- hand the denominators to the lanes that hold the matching accumulator rows, then store ----
+    waveLdsFence();
+#pragma unroll
+    for (int g = 0; g < GC; ++g) {
+        if (lane == 0) statW[g] = lRun[g];
+    }
+    waveLdsFence();
+    const bool single = L <= sp.TT;  // the whole sequence lives in this range
+    const int64_t split = blockIdx.y;
+    if (!single && lane < G) {
+        // lane g publishes (max, denominator) of query head g
+        float mg = -INFINITY;
+#pragma unroll
+        for (int g = 0; g < GC; ++g) mg = (lane == g) ? mRun[g] : mg;
+        float* ml = sp.partMl + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + hk * G + lane) * 2;
+        ml[0] = mg;
+        ml[1] = statW[lane];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int g = 4 * q + r;
+        if (g >= G) continue;
+        const int qh = hk * G + g;
+        if (single) {
+            const float inv = 1.f / statW[g];
+            Pack16<T> o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.e[e] = static_cast<T>(acc[e][r] * inv);
+            storePack(out + (static_cast<int64_t>(i) * a.H + qh) * kD + c * 8, o);
+        } else {
+            float* dst = sp.partAcc + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * kD + c * 8;
+            *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
         }
     }
 }
@@ -545,31 +392,17 @@ __global__ __launch_bounds__(kRvThreads) void softmaxReduceVGeneric(T* __restric
     }
 }
 
-int pow2Floor(int x) {
-    int p = 1;
-    while (p * 2 <= x) p *= 2;
-    return p;
-}
-
 template <typename T>
-diopiError_t launchSplit(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* logits, const void* v, const DecodeArgs& a) {
+diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* logits, const void* v, const DecodeArgs& a) {
     SplitArgs sp;
-    // Range length: the fp32 partial of a range (G*D*4 bytes per kv head) should stay near 1.5 % of the
-    // V bytes the range streams (TT*D*2 per kv head)  =>  TT >= ~128*G; heads per group then chosen so
-    // that a work-group streams roughly half a MiB.
+    // tokens per range: the fp32 partial (G*D*4 bytes per kv head) against the V bytes it summarises (TT*D*2): about
+    // 1.5 % at TT = 128*G; shorter ranges balance ragged batches better, longer ones amortise the pipeline start
     int TT = 128 * a.G;
     if (TT < 512) TT = 512;
     if (TT > 2048) TT = 2048;
     TT = envInt("DIOPI_ROCM_REDUCEV_TT", TT);
     TT = static_cast<int>(ceilDiv(TT, kSub)) * kSub;
-    int HB = pow2Floor(static_cast<int>((512 * 1024) / (static_cast<int64_t>(TT) * kD * sizeof(T))));
-    if (HB > 16) HB = 16;
-    if (HB < 1) HB = 1;
-    while (HB > 1 && HB * a.G > kMaxHeadsQ) HB /= 2;
-    while (HB > 1 && HB > pow2Floor(a.Hkv) ) HB /= 2;
-    HB = envInt("DIOPI_ROCM_REDUCEV_HB", HB);
     sp.TT = TT;
-    sp.HB = HB;
     sp.splits = static_cast<int>(ceilDiv(a.maxInputLen, TT));
     sp.partAcc = nullptr;
     sp.partMl = nullptr;
@@ -581,55 +414,23 @@ diopiError_t launchSplit(diopiContextHandle_t ctx, hipStream_t stream, void* out
         sp.partAcc = static_cast<float*>(scratch);
         sp.partMl = reinterpret_cast<float*>(static_cast<char*>(scratch) + accBytes);
     }
-    const dim3 grid(static_cast<unsigned>(sp.splits), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.Hkv, HB)));
-#define ROCM_RV_CASE(GC)                                                                                                                       \
-    hipLaunchKernelGGL((softmaxReduceVSplit<T, GC>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
+    ROCM_CHECK(sp.splits <= 65535, "max_input_len %d needs more than 65535 ranges of %d tokens", a.maxInputLen, TT);
+    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits), static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves)));
+#define ROCM_RVW_CASE(GC)                                                                                                                   \
+    hipLaunchKernelGGL((softmaxReduceVWave<T, GC>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
                        static_cast<const T*>(v), a, sp)
-    switch (a.G) {
-        case 1: ROCM_RV_CASE(1); break;
-        case 2: ROCM_RV_CASE(2); break;
-        case 4: ROCM_RV_CASE(4); break;
-        case 8: ROCM_RV_CASE(8); break;
-        default: ROCM_CHECK(false, "unsupported group size %d in the split kernel", a.G);
+    if (a.G <= 1) {
+        ROCM_RVW_CASE(1);
+    } else if (a.G <= 2) {
+        ROCM_RVW_CASE(2);
+    } else if (a.G <= 4) {
+        ROCM_RVW_CASE(4);
+    } else if (a.G <= 8) {
+        ROCM_RVW_CASE(8);
+    } else {
+        ROCM_RVW_CASE(16);
     }
-#undef ROCM_RV_CASE
-    ROCM_LAUNCH_CHECK();
-    if (sp.splits > 1) {
-        const dim3 mgrid(static_cast<unsigned>(ceilDiv(static_cast<int64_t>(a.H) * a.D, kRvThreads)), static_cast<unsigned>(a.batch));
-        hipLaunchKernelGGL(softmaxReduceVMerge<T>, mgrid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), a, sp);
-        ROCM_LAUNCH_CHECK();
-    }
-    return diopiSuccess;
-}
-
-template <typename T>
-diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* logits, const void* v, const DecodeArgs& a) {
-    SplitArgs sp;
-    // tokens per partial: the fp32 partial (G*D*4 bytes) against the V bytes it summarises (TT*D*2): about 1.5 % at TT = 128*G
-    int TT = 128 * a.G;
-    if (TT < 512) TT = 512;
-    if (TT > 4096) TT = 4096;
-    TT = envInt("DIOPI_ROCM_REDUCEV_TT", TT);
-    TT = static_cast<int>(ceilDiv(TT, kVTileTokens)) * kVTileTokens;
-    // one kv head per wave; with fewer than four kv heads the spare waves take further token ranges
-    const int HS = a.Hkv >= 4 ? 4 : (a.Hkv >= 2 ? 2 : 1);
-    const int TPH = kRvWaves / HS;
-    sp.TT = TT;
-    sp.HB = HS;
-    sp.splits = static_cast<int>(ceilDiv(a.maxInputLen, TT));
-    sp.partAcc = nullptr;
-    sp.partMl = nullptr;
-    if (sp.splits > 1) {
-        const int64_t accBytes = static_cast<int64_t>(a.batch) * sp.splits * a.H * kD * sizeof(float);
-        const int64_t mlBytes = static_cast<int64_t>(a.batch) * sp.splits * a.H * 2 * sizeof(float);
-        void* scratch = nullptr;
-        ROCM_CALL(requireScratch(ctx, accBytes + mlBytes, &scratch));
-        sp.partAcc = static_cast<float*>(scratch);
-        sp.partMl = reinterpret_cast<float*>(static_cast<char*>(scratch) + accBytes);
-    }
-    const dim3 grid(static_cast<unsigned>(ceilDiv(sp.splits, TPH)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.Hkv, HS)));
-    hipLaunchKernelGGL(softmaxReduceVMfma<T>, grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits),
-                       static_cast<const T*>(v), a, sp, HS);
+#undef ROCM_RVW_CASE
     ROCM_LAUNCH_CHECK();
     if (sp.splits > 1) {
         const dim3 mgrid(static_cast<unsigned>(ceilDiv(static_cast<int64_t>(a.H) * a.D, kRvThreads)), static_cast<unsigned>(a.batch));
@@ -671,21 +472,15 @@ extern "C" diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t c
 
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    const bool fast = a.D == kD && (a.G == 1 || a.G == 2 || a.G == 4 || a.G == 8) && (reinterpret_cast<uintptr_t>(vV.data) & 15) == 0 &&
-                      envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
-    // The vector-ALU split kernel is instantiated for G in {1, 2, 4, 8}; other group sizes up to 16 (and any G at or
-    // above DIOPI_ROCM_REDUCEV_MFMA_MIN_G) take the MFMA kernel.
-    const int mfmaMinG = envInt("DIOPI_ROCM_REDUCEV_MFMA_MIN_G", 17);
-    const bool mfma = a.D == kD && a.G <= 16 && (a.G >= mfmaMinG || !fast) && (reinterpret_cast<uintptr_t>(vV.data) & 15) == 0 &&
+    // the matrix-core kernel keeps slot numbers in 32 bits and reads V rows with 16-byte loads
+    const bool mfma = a.D == kD && a.G <= 16 && a.numSlots < (int64_t(1) << 31) && (reinterpret_cast<uintptr_t>(vV.data) & 15) == 0 &&
                       envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
     switch (vOut.dtype) {
         case diopi_dtype_float16:
-            if (mfma) return launchMfma<half_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a);
-            return fast ? launchSplit<half_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)
+            return mfma ? launchWave<half_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)
                         : launchGeneric<half_t, float>(stream, vOut.data, vLogits.data, vV.data, a);
         case diopi_dtype_bfloat16:
-            if (mfma) return launchMfma<bf16_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a);
-            return fast ? launchSplit<bf16_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)
+            return mfma ? launchWave<bf16_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)
                         : launchGeneric<bf16_t, float>(stream, vOut.data, vLogits.data, vV.data, a);
         case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vLogits.data, vV.data, a);
         case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vLogits.data, vV.data, a);
