@@ -34,7 +34,10 @@ constexpr int kBM = 128;   // query rows per work-group
 constexpr int kBN = 64;    // key rows per tile
 constexpr int kHD = 128;   // head size of the MFMA kernel
 constexpr int kLD = kHD + 8;  // LDS row pitch in elements (272 bytes: 16-byte aligned, conflict-free 128-bit reads)
+constexpr int kVP = kBN + 8;   // row pitch of the transposed V tile in elements (144 bytes)
+constexpr int kStageElems = kBN * kLD + kHD * kVP;  // one staging buffer (K tile + transposed V tile), in elements
 constexpr int kNumXcd = 8;
+constexpr float kLazyLog2 = 8.0f;  // how far (in powers of two) the softmax reference maximum may lag behind
 
 struct CtxArgs {
     const void* bStartLoc;
@@ -43,6 +46,8 @@ struct CtxArgs {
     int batch;
     int H;
     int64_t rows;      // rows of q / k / v / out
+    int dbg = 0;
+    const int2* plan;  // [tilesBound] visiting order of the query tiles of one head, written by ctxAttnPlan
     int tilesBound;    // upper bound on the number of 128-row query tiles over all sequences
     int totalItems;    // H * tilesBound
 };
@@ -83,14 +88,54 @@ __device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
     return s;
 }
 
+// Visiting order of the query tiles of one head: entry p of `plan` is (sequence, query tile index), sorted by tile
+// index descending.  A query tile with index t attends to t + 1 key blocks, so this is longest-job-first and the
+// short tiles fill the tail of the launch whatever the mix of sequence lengths.  With the sequences ranked by tile
+// count (descending), the sequences that own a tile of index t are a prefix of that ranking, hence
+//   position(seq, t) = sum_s max(0, tiles_s - 1 - t)  +  rank(seq).
+// One work-group; tile counts are kept in LDS.  Unused entries (the bound over-counts) get sequence -1.
+constexpr int kPlanThreads = 1024;
+__global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ plan, CtxArgs a, int maxTiles) {
+    extern __shared__ int sTiles[];  // [batch]
+    const int tid = threadIdx.x;
+    for (int s = tid; s < a.batch; s += kPlanThreads) sTiles[s] = static_cast<int>((loadSeq(a, s).len + kBM - 1) / kBM);
+    for (int p = tid; p < a.tilesBound; p += kPlanThreads) plan[p] = make_int2(-1, 0);
+    __syncthreads();
+    for (int s = tid; s < a.batch; s += kPlanThreads) {
+        const int nt = sTiles[s];
+        if (nt == 0) continue;
+        int rank = 0;
+        for (int s2 = 0; s2 < a.batch; ++s2) {
+            const int nt2 = sTiles[s2];
+            rank += (nt2 > nt || (nt2 == nt && s2 < s)) ? 1 : 0;
+        }
+        sTiles[a.batch + s] = rank;
+    }
+    __syncthreads();
+    for (int t = tid; t < maxTiles; t += kPlanThreads) {
+        int off = 0;
+        for (int s = 0; s < a.batch; ++s) {
+            const int more = sTiles[s] - 1 - t;
+            off += more > 0 ? more : 0;
+        }
+        sTiles[2 * a.batch + t] = off;
+    }
+    __syncthreads();
+    for (int s = 0; s < a.batch; ++s) {
+        const int nt = sTiles[s];
+        const int rank = nt > 0 ? sTiles[a.batch + s] : 0;
+        for (int t = tid; t < nt; t += kPlanThreads) plan[sTiles[2 * a.batch + t] + rank] = make_int2(s, t);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                                                CtxArgs a, float scaleLog2) {
     using Ops = Mfma32<T>;
     using Frag = typename Ops::Frag;
-    __shared__ __attribute__((aligned(16))) T smem[2 * kBN * kLD];
-    T* sK = smem;
-    T* sV = smem + kBN * kLD;
+    // two staging buffers of (K tile [key][dim] row-major, V tile transposed [dim row][key position], see below)
+    extern __shared__ __attribute__((aligned(16))) unsigned char dynSmem[];
+    T* smem = reinterpret_cast<T*>(dynSmem);
 
     // ---- which (head, sequence, query tile) is this work-group? ----
     const int perXcd = (a.totalItems + kNumXcd - 1) / kNumXcd;
@@ -98,18 +143,12 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     if (item >= a.totalItems) return;
     const int head = item / a.tilesBound;
     const int tileFlat = item % a.tilesBound;
-    int seq = 0, before = 0, numTiles = 0;
-    SeqInfo si{0, 0};
-    for (; seq < a.batch; ++seq) {
-        si = loadSeq(a, seq);
-        numTiles = static_cast<int>((si.len + kBM - 1) / kBM);
-        if (tileFlat < before + numTiles) break;
-        before += numTiles;
-    }
-    if (seq >= a.batch) return;
-    const int qt = numTiles - 1 - (tileFlat - before);  // last (longest) tiles first
-    const int64_t L = si.len;
-    const int64_t m0 = static_cast<int64_t>(qt) * kBM;
+    const int2 planned = a.plan[tileFlat];  // (sequence, query tile), longest tiles first; sequence -1 = padding
+    if (planned.x < 0) return;
+    const int qt = planned.y;
+    const SeqInfo si = loadSeq(a, planned.x);
+    const int L = static_cast<int>(si.len);              // the launcher checked that row counts fit 32 bits
+    const int m0 = qt * kBM;
 
     const int tid = threadIdx.x;
     const int lane = tid % kWave;
@@ -122,8 +161,8 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
 
     // ---- Q fragments (B operand of S^T): row = m0 + 32*wave + n, k slot (hh, e) <-> dim 16*s + 8*hh + e ----
-    const int64_t qRow = m0 + wave * 32 + n;
-    const int64_t qRowLd = qRow < L ? qRow : L - 1;
+    const int qRow = m0 + wave * 32 + n;
+    const int qRowLd = qRow < L ? qRow : L - 1;
     Frag qf[kHD / 16];
 #pragma unroll
     for (int s = 0; s < kHD / 16; ++s) {
@@ -141,59 +180,112 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     float mRun = -1e30f;
     float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
 
-    const int64_t kEnd = (m0 + kBM < L) ? m0 + kBM : L;  // keys 0 .. kEnd-1 are visible to this tile
-    const int numKeyTiles = static_cast<int>((kEnd + kBN - 1) / kBN);
-    const int64_t waveRowLo = m0 + wave * 32;
-    const int64_t waveRowHi = waveRowLo + 31;
+    const int kEnd = (m0 + kBM < L) ? m0 + kBM : L;  // keys 0 .. kEnd-1 are visible to this tile
+    const int numKeyTiles = (kEnd + kBN - 1) / kBN;
+    const int waveRowLo = m0 + wave * 32;
+    const int waveRowHi = waveRowLo + 31;
 
-    // tile staging: thread -> 16-byte packet ldC of rows ldR, ldR+16, ldR+32, ldR+48
+    // ---- tile staging ----
+    // K: thread -> 16-byte packet ldC of rows ldR, ldR+16, ldR+32, ldR+48, stored as they are.
+    // V: stored transposed, sVt[row(dim)][position(key)], so that the A operand of the second product (8 keys of one
+    //    dim) is one 16-byte read.  A thread takes packet ldC (dims 8*ldC .. +7) of two adjacent keys, interleaves
+    //    them with byte permutes and writes one dword (key pair) per dim.  The row of dim 8*c + e is 16*e + c and
+    //    the keys of a 16-key group sit in the order (0-3, 8-11, 4-7, 12-15): with the 144-byte row pitch this makes
+    //    both the dword writes and the 16-byte reads free of bank conflicts, and the key order matches the k slots in
+    //    which the first product leaves the probabilities (lane half hh owns keys 4*hh + {0..3, 8..11} of a group).
     const int ldC = tid % 16;
     const int ldR = tid / 16;
-    u32x4 kReg[4], vReg[4];
+    const int q4 = lane / 16;
+    u32x4 kReg[4], vReg[2][2];
     auto loadTile = [&](int jt) {
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-            int64_t row = static_cast<int64_t>(jt) * kBN + ldR + it * 16;
-            if (row > L - 1) row = L - 1;  // keeps the load in bounds; such keys are masked below
+            int row = jt * kBN + ldR + it * 16;
+            row = row < L ? row : L - 1;  // keeps the load in bounds; such keys are masked below
             kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
-            vReg[it] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                int row = jt * kBN + 16 * wave + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * it + h2;
+                row = row < L ? row : L - 1;
+                vReg[it][h2] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
+            }
+        }
+    };
+    auto stageTile = [&](int buf) {
+        T* sK = smem + buf * kStageElems;
+        uint32_t* sVt32 = reinterpret_cast<uint32_t*>(sK + kBN * kLD);
+#pragma unroll
+        for (int it = 0; it < 4; ++it) *reinterpret_cast<u32x4*>(sK + (ldR + it * 16) * kLD + ldC * 8) = kReg[it];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int posd = 8 * wave + 4 * it + q4;  // dword position of this key pair inside a row
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t pair = __builtin_amdgcn_perm(vReg[it][1][e / 2], vReg[it][0][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
+                sVt32[(16 * e + ldC) * (kVP / 2) + posd] = pair;
+            }
         }
     };
     loadTile(0);
+    stageTile(0);
+    if (numKeyTiles > 1) loadTile(1);
 
     for (int jt = 0; jt < numKeyTiles; ++jt) {
-        __syncthreads();  // every wave is done with the previous tile
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            *reinterpret_cast<u32x4*>(sK + (ldR + it * 16) * kLD + ldC * 8) = kReg[it];
-            *reinterpret_cast<u32x4*>(sV + (ldR + it * 16) * kLD + ldC * 8) = vReg[it];
+        // One barrier per tile: tile jt is staged and every wave has left tile jt-1, whose buffer now takes tile
+        // jt+1 (requested one iteration ago, so its latency is covered); the request for tile jt+2 follows.
+        if (!(a.dbg & 16)) __syncthreads();
+        if (!(a.dbg & 1)) {
+            if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
+            if (jt + 2 < numKeyTiles) loadTile(jt + 2);
         }
-        __syncthreads();
-        if (jt + 1 < numKeyTiles) loadTile(jt + 1);  // in flight while this tile is computed
+        const T* sK = smem + (jt & 1) * kStageElems;
+        const T* sVt = sK + kBN * kLD;
 
-        const int64_t key0 = static_cast<int64_t>(jt) * kBN;
+        const int key0 = jt * kBN;
         if (key0 > waveRowHi) continue;  // entirely above the diagonal for this wave (barriers are at the loop top)
 
         // ---- S^T = K . Q^T for the two 32-key blocks ----
+        // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
+        // alternate so that consecutive products never wait on each other's accumulator.
         f32x16 s[2];
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
-#pragma unroll
-            for (int st = 0; st < kHD / 16; ++st) {
-                FragBits<Frag> u;
-                u.raw = *reinterpret_cast<const u32x4*>(sK + (sb * 32 + n) * kLD + st * 16 + hh * 8);
-                s[sb] = Ops::mma(u.f, qf[st], s[sb]);
-            }
         }
+        FragBits<Frag> kf[2][2];
+        auto loadK = [&](int st, int b) {
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb) kf[b][sb].raw = *reinterpret_cast<const u32x4*>(sK + (sb * 32 + n) * kLD + st * 16 + hh * 8);
+        };
+        loadK(0, 0);
+        if (!(a.dbg & 2))
+#pragma unroll
+        for (int st = 0; st < kHD / 16; ++st) {
+            if (st + 1 < kHD / 16) loadK(st + 1, (st + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the read-ahead order: the scheduler would otherwise sink the reads
+            s[0] = Ops::mma(kf[st & 1][0].f, qf[st], s[0]);
+            s[1] = Ops::mma(kf[st & 1][1].f, qf[st], s[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // V^T operands of the first 16-key group travel while the softmax runs
+        FragBits<Frag> vf[2][kHD / 32];
+        auto loadV = [&](int g, int b) {
+#pragma unroll
+            for (int mb = 0; mb < kHD / 32; ++mb) vf[b][mb].raw = *reinterpret_cast<const u32x4*>(sVt + (32 * mb + n) * kVP + 16 * g + 8 * hh);
+        };
+        loadV(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
         // accumulator register r of block sb holds key  key0 + 32*sb + 8*(r/4) + 4*hh + r%4  for query row qRow
         if (key0 + kBN - 1 > waveRowLo) {
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int64_t key = key0 + sb * 32 + (r / 4) * 8 + hh * 4 + (r % 4);
+                    const int key = key0 + sb * 32 + (r / 4) * 8 + hh * 4 + (r % 4);
                     if (key > qRow) s[sb][r] = -1e30f;
                 }
             }
@@ -205,11 +297,22 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
             for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[sb][r]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-        const float mNew = fmaxf(mRun, tmax);
-        const float alpha = __builtin_amdgcn_exp2f((mRun - mNew) * scaleLog2);
-        const float mc = mNew * scaleLog2;
-        mRun = mNew;
-        float psum = 0.f;
+        // The reference maximum only follows the true one when it has fallen behind by more than 2^kLazyLog2 (a
+        // wave-uniform, rarely taken branch after the first tiles): probabilities then reach at most 2^kLazyLog2,
+        // which the 16-bit types hold with full relative precision, and the accumulators are rescaled only then.
+        if (__any((tmax - mRun) * scaleLog2 > kLazyLog2)) {
+            const float mNew = fmaxf(mRun, tmax);
+            const float alpha = __builtin_amdgcn_exp2f((mRun - mNew) * scaleLog2);
+            mRun = mNew;
+            lRun *= alpha;
+#pragma unroll
+            for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[mb][r] *= alpha;
+            }
+        }
+        const float mc = mRun * scaleLog2;
+        float psum[4] = {0.f, 0.f, 0.f, 0.f};
         Frag pf[2][2];
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
@@ -217,34 +320,23 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
-                    psum += p;
+                    const float p = (a.dbg & 4) ? s[sb][u * 8 + j] : __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
+                    psum[j & 3] += p;
                     pf[sb][u][j] = static_cast<T>(p);
                 }
             }
         }
-        lRun = lRun * alpha + psum;
+        lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
+        // ---- O^T += V^T . P^T : k slot (hh, j) of group g = 2*sb + u is key 16*g + 8*(j/4) + 4*hh + j%4 ----
+        // accumulator row n' of o[mb] stands for LDS row 32*mb + n', i.e. dim 8 * (row % 16) + row / 16
+        if (!(a.dbg & 8))
 #pragma unroll
-        for (int mb = 0; mb < kHD / 32; ++mb) {
+        for (int g = 0; g < 4; ++g) {
+            if (g + 1 < 4) loadV(g + 1, (g + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[mb][r] *= alpha;
-        }
-        // ---- O^T += V^T . P^T : k slot (hh, j) of step (sb, u) is key 32*sb + 16*u + 8*(j/4) + 4*hh + j%4 ----
-#pragma unroll
-        for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-#pragma unroll
-                for (int mb = 0; mb < kHD / 32; ++mb) {
-                    Frag vf;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int key = sb * 32 + u * 16 + (j / 4) * 8 + hh * 4 + (j % 4);
-                        vf[j] = sV[key * kLD + mb * 32 + n];
-                    }
-                    o[mb] = Ops::mma(vf, pf[sb][u], o[mb]);
-                }
-            }
+            for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -253,25 +345,28 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     const float inv = 1.0f / lTot;
     __syncthreads();  // the K/V tiles are dead; reuse the storage as a [128][kLD] output tile
     T* sO = smem;
+    static_assert(kBM * kLD <= 2 * kStageElems, "the output tile must fit the staging storage");
 #pragma unroll
     for (int mb = 0; mb < kHD / 32; ++mb) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            // registers 4*r4 .. 4*r4+3 are dims 32*mb + 8*r4 + 4*hh + 0..3 of query row (32*wave + n)
-            T pk[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) pk[e] = static_cast<T>(o[mb][r4 * 4 + e] * inv);
-            *reinterpret_cast<u32x2*>(sO + (wave * 32 + n) * kLD + mb * 32 + r4 * 8 + hh * 4) = *reinterpret_cast<const u32x2*>(pk);
+        for (int r = 0; r < 8; ++r) {
+            // registers r and r + 8 of o[mb] are LDS rows 32*mb + 8*(r/4) + 4*hh + r%4 (+16): dims d and d + 1
+            const int d = 64 * ((r >> 2) & 1) + 32 * hh + 8 * (r & 3) + 2 * mb;
+            T pk[2];
+            pk[0] = static_cast<T>(o[mb][r] * inv);
+            pk[1] = static_cast<T>(o[mb][r + 8] * inv);
+            *reinterpret_cast<uint32_t*>(sO + (wave * 32 + n) * kLD + d) = *reinterpret_cast<const uint32_t*>(pk);
         }
     }
     // each wave only reads back the 32 rows it wrote: no work-group barrier needed, LDS ops of a wave are ordered
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     T* oBase = out + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
         const int id = it * kWave + lane;
         const int row = id / 16;
         const int c = id % 16;
-        const int64_t grow = m0 + wave * 32 + row;
+        const int grow = m0 + wave * 32 + row;
         if (grow < L) {
             const u32x4 val = *reinterpret_cast<const u32x4*>(sO + (wave * 32 + row) * kLD + c * 8);
             *reinterpret_cast<u32x4*>(oBase + grow * rowPitch + c * 8) = val;
@@ -336,15 +431,27 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
 }
 
 template <typename T>
-diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
+diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
+    a.dbg = envInt("DIOPI_ROCM_CTX_DBG", 0);
     a.tilesBound = static_cast<int>(ceilDiv(a.rows, kBM)) + a.batch;
     const int64_t total = static_cast<int64_t>(a.tilesBound) * a.H;
     ROCM_CHECK(total < INT32_MAX / 2, "context attention: too many tiles for one launch");
     a.totalItems = static_cast<int>(total);
+    // visiting order of the query tiles (context-owned scratch, rebuilt by every call on the device)
+    void* planMem = nullptr;
+    ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int2), &planMem));
+    a.plan = static_cast<const int2*>(planMem);
+    const int maxTiles = static_cast<int>(ceilDiv(a.rows, kBM));
+    const size_t planLds = (2 * static_cast<size_t>(a.batch) + maxTiles) * sizeof(int);
+    hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles);
+    ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
     // exp(x) = exp2(x * log2(e)); the 1/sqrt(D) scaling of the scores is folded into the same factor
     const float scaleLog2 = static_cast<float>(1.4426950408889634 / std::sqrt(static_cast<double>(kHD)));
-    hipLaunchKernelGGL(ctxAttnMfma<T>, dim3(grid), dim3(kCtxThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
+    constexpr int ldsBytes = 2 * kStageElems * static_cast<int>(sizeof(T));
+    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+    ROCM_HIP(granted);
+    hipLaunchKernelGGL(ctxAttnMfma<T>, dim3(grid), dim3(kCtxThreads), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
                        static_cast<const T*>(v), a, scaleLog2);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
@@ -409,13 +516,15 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     ROCM_CALL(getStream(ctx, &stream));
     const bool aligned =
         ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
-    const bool fast = D == kHD && aligned && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    // the planning kernel keeps two ints per sequence and one per query tile in LDS
+    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBM + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
+    const bool fast = D == kHD && aligned && planFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
     switch (vQ.dtype) {
         case diopi_dtype_float16:
-            return fast ? launchMfma<half_t>(stream, vOut.data, vQ.data, vK.data, vV.data, a)
+            return fast ? launchMfma<half_t>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
                         : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_bfloat16:
-            return fast ? launchMfma<bf16_t>(stream, vOut.data, vQ.data, vK.data, vV.data, a)
+            return fast ? launchMfma<bf16_t>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
                         : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
