@@ -10,17 +10,21 @@
 // probabilities, which stays inside the reference's 16-bit tolerance.  Rows outside every sequence
 // are not written; max_input_len is not needed (the reference never reads it either).
 //
-// MFMA kernel (fp16 / bf16, D == 128).  One 256-thread work-group owns 128 query rows of one
-// (sequence, head); each of its four waves owns 32 of them.  Key/value tiles of 64 rows are staged
-// row-major in LDS and shared by the four waves.  Everything is computed transposed so that no
-// cross-lane data movement is needed between the two matrix products:
+// MFMA kernel (fp16 / bf16, D == 128).  A work-group of 4 or 8 waves owns 128 or 256 query rows of one
+// (sequence, head); each wave owns 32 of them.  Key/value tiles of 64 rows are staged in LDS (two buffers, one
+// barrier per tile, the global request for a tile is issued a whole iteration before it is needed) and shared by
+// the waves.  Everything is computed transposed so that no cross-lane data movement is needed between the two
+// matrix products:
 //   S^T[key, q]  = K[key, :] . Q[q, :]      v_mfma_f32_32x32x16, A = K rows from LDS, B = Q rows (registers)
-//   O^T[d, q]   += V^T[d, key] . P^T[key, q]                    A = V columns from LDS, B = P^T
-// In the 32x32 accumulator layout a lane holds one query column, so the row maximum, the row sum
-// and the rescaling of O^T are per-lane scalars (one exchange with lane ^ 32 per tile), and the
-// exponentiated scores are already in the B-operand layout of the second product.
-// Work-groups are numbered so that the query tiles of one head land on the same XCD (they share
-// that head's K/V through its L2), and the heaviest (last) query tiles of a sequence start first.
+//   O^T[d, q]   += V^T[d, key] . P^T[key, q]                    A = V^T rows from LDS, B = P^T
+// In the 32x32 accumulator layout a lane holds one query column, so the row maximum, the row sum and the rescaling
+// of O^T are per-lane scalars (one exchange with lane ^ 32 per tile), and the exponentiated scores are already in
+// the B-operand layout of the second product.  The V tile is transposed once, when it is staged (byte permutes on
+// key pairs, dword writes), so that the second product's A operand is a single 16-byte LDS read like the first's.
+// The softmax reference maximum is updated lazily (only when it lags by more than 2^8), which keeps the rescaling
+// of the 64 accumulator registers out of the common path.
+// Work-groups are numbered so that the query tiles of one head land on the same XCD (they share that head's K/V
+// through its L2); a small planning kernel orders the tiles of a head longest first.
 #include <cmath>
 
 #include "common.hpp"
@@ -29,8 +33,7 @@
 namespace rocm {
 namespace {
 
-constexpr int kCtxThreads = 256;
-constexpr int kBM = 128;   // query rows per work-group
+constexpr int kBMMin = 128;  // smallest query tile of a work-group (bounds of the planning step are sized for it)
 constexpr int kBN = 64;    // key rows per tile
 constexpr int kHD = 128;   // head size of the MFMA kernel
 constexpr int kLD = kHD + 8;  // LDS row pitch in elements (272 bytes: 16-byte aligned, conflict-free 128-bit reads)
@@ -46,7 +49,6 @@ struct CtxArgs {
     int batch;
     int H;
     int64_t rows;      // rows of q / k / v / out
-    int dbg = 0;
     const int2* plan;  // [tilesBound] visiting order of the query tiles of one head, written by ctxAttnPlan
     int tilesBound;    // upper bound on the number of 128-row query tiles over all sequences
     int totalItems;    // H * tilesBound
@@ -95,10 +97,10 @@ __device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
 //   position(seq, t) = sum_s max(0, tiles_s - 1 - t)  +  rank(seq).
 // One work-group; tile counts are kept in LDS.  Unused entries (the bound over-counts) get sequence -1.
 constexpr int kPlanThreads = 1024;
-__global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ plan, CtxArgs a, int maxTiles) {
+__global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ plan, CtxArgs a, int maxTiles, int bm) {
     extern __shared__ int sTiles[];  // [batch]
     const int tid = threadIdx.x;
-    for (int s = tid; s < a.batch; s += kPlanThreads) sTiles[s] = static_cast<int>((loadSeq(a, s).len + kBM - 1) / kBM);
+    for (int s = tid; s < a.batch; s += kPlanThreads) sTiles[s] = static_cast<int>((loadSeq(a, s).len + bm - 1) / bm);
     for (int p = tid; p < a.tilesBound; p += kPlanThreads) plan[p] = make_int2(-1, 0);
     __syncthreads();
     for (int s = tid; s < a.batch; s += kPlanThreads) {
@@ -128,11 +130,13 @@ __global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ p
     }
 }
 
-template <typename T>
-__global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+template <typename T, int NWV>
+__global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                                                CtxArgs a, float scaleLog2) {
     using Ops = Mfma32<T>;
     using Frag = typename Ops::Frag;
+    constexpr int BM = NWV * 32;  // query rows per work-group: each of the NWV waves owns 32 of them
+    constexpr int kThreads = NWV * kWave;
     // two staging buffers of (K tile [key][dim] row-major, V tile transposed [dim row][key position], see below)
     extern __shared__ __attribute__((aligned(16))) unsigned char dynSmem[];
     T* smem = reinterpret_cast<T*>(dynSmem);
@@ -148,7 +152,7 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     const int qt = planned.y;
     const SeqInfo si = loadSeq(a, planned.x);
     const int L = static_cast<int>(si.len);              // the launcher checked that row counts fit 32 bits
-    const int m0 = qt * kBM;
+    const int m0 = qt * BM;
 
     const int tid = threadIdx.x;
     const int lane = tid % kWave;
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     float mRun = -1e30f;
     float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
 
-    const int kEnd = (m0 + kBM < L) ? m0 + kBM : L;  // keys 0 .. kEnd-1 are visible to this tile
+    const int kEnd = (m0 + BM < L) ? m0 + BM : L;  // keys 0 .. kEnd-1 are visible to this tile
     const int numKeyTiles = (kEnd + kBN - 1) / kBN;
     const int waveRowLo = m0 + wave * 32;
     const int waveRowHi = waveRowLo + 31;
@@ -196,19 +200,23 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     const int ldC = tid % 16;
     const int ldR = tid / 16;
     const int q4 = lane / 16;
-    u32x4 kReg[4], vReg[2][2];
+    constexpr int kRowsPerPass = kThreads / 16;         // K rows covered by one pass of the work-group
+    constexpr int kKPasses = kBN / kRowsPerPass;        // 4 (256 threads) or 2 (512 threads)
+    constexpr int kVItems = (kBN / 2) * 16 / kThreads;  // (key pair, packet) items per thread: 2 or 1
+    u32x4 kReg[kKPasses], vReg[kVItems][2];
     auto loadTile = [&](int jt) {
 #pragma unroll
-        for (int it = 0; it < 4; ++it) {
-            int row = jt * kBN + ldR + it * 16;
+        for (int it = 0; it < kKPasses; ++it) {
+            int row = jt * kBN + ldR + it * kRowsPerPass;
             row = row < L ? row : L - 1;  // keeps the load in bounds; such keys are masked below
             kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
         }
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
+        for (int it = 0; it < kVItems; ++it) {
+            const int ci = wave * kVItems + it;  // 0..7: 16-key group ci / 2, half ci % 2
 #pragma unroll
             for (int h2 = 0; h2 < 2; ++h2) {
-                int row = jt * kBN + 16 * wave + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * it + h2;
+                int row = jt * kBN + 16 * (ci / 2) + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * (ci % 2) + h2;
                 row = row < L ? row : L - 1;
                 vReg[it][h2] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
             }
@@ -218,10 +226,11 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
         T* sK = smem + buf * kStageElems;
         uint32_t* sVt32 = reinterpret_cast<uint32_t*>(sK + kBN * kLD);
 #pragma unroll
-        for (int it = 0; it < 4; ++it) *reinterpret_cast<u32x4*>(sK + (ldR + it * 16) * kLD + ldC * 8) = kReg[it];
+        for (int it = 0; it < kKPasses; ++it) *reinterpret_cast<u32x4*>(sK + (ldR + it * kRowsPerPass) * kLD + ldC * 8) = kReg[it];
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            const int posd = 8 * wave + 4 * it + q4;  // dword position of this key pair inside a row
+        for (int it = 0; it < kVItems; ++it) {
+            const int ci = wave * kVItems + it;
+            const int posd = 8 * (ci / 2) + 4 * (ci % 2) + q4;  // dword position of this key pair inside a row
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t pair = __builtin_amdgcn_perm(vReg[it][1][e / 2], vReg[it][0][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
@@ -236,16 +245,17 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
     for (int jt = 0; jt < numKeyTiles; ++jt) {
         // One barrier per tile: tile jt is staged and every wave has left tile jt-1, whose buffer now takes tile
         // jt+1 (requested one iteration ago, so its latency is covered); the request for tile jt+2 follows.
-        if (!(a.dbg & 16)) __syncthreads();
-        if (!(a.dbg & 1)) {
-            if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
-            if (jt + 2 < numKeyTiles) loadTile(jt + 2);
-        }
+        __syncthreads();
         const T* sK = smem + (jt & 1) * kStageElems;
         const T* sVt = sK + kBN * kLD;
 
         const int key0 = jt * kBN;
-        if (key0 > waveRowHi) continue;  // entirely above the diagonal for this wave (barriers are at the loop top)
+        if (key0 > waveRowHi) {
+            // entirely above the diagonal for this wave: only the staging duty remains
+            if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
+            if (jt + 2 < numKeyTiles) loadTile(jt + 2);
+            continue;
+        }  // entirely above the diagonal for this wave (barriers are at the loop top)
 
         // ---- S^T = K . Q^T for the two 32-key blocks ----
         // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
@@ -256,19 +266,20 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
         }
-        FragBits<Frag> kf[2][2];
+        constexpr int kKDepth = 2;  // K operand steps in flight: LDS latency under load spans several products
+        FragBits<Frag> kf[kKDepth][2];
         auto loadK = [&](int st, int b) {
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb) kf[b][sb].raw = *reinterpret_cast<const u32x4*>(sK + (sb * 32 + n) * kLD + st * 16 + hh * 8);
         };
-        loadK(0, 0);
-        if (!(a.dbg & 2))
+#pragma unroll
+        for (int st = 0; st < kKDepth - 1; ++st) loadK(st, st);
 #pragma unroll
         for (int st = 0; st < kHD / 16; ++st) {
-            if (st + 1 < kHD / 16) loadK(st + 1, (st + 1) & 1);
+            if (st + kKDepth - 1 < kHD / 16) loadK(st + kKDepth - 1, (st + kKDepth - 1) % kKDepth);
             __builtin_amdgcn_sched_barrier(0);  // keep the read-ahead order: the scheduler would otherwise sink the reads
-            s[0] = Ops::mma(kf[st & 1][0].f, qf[st], s[0]);
-            s[1] = Ops::mma(kf[st & 1][1].f, qf[st], s[1]);
+            s[0] = Ops::mma(kf[st % kKDepth][0].f, qf[st], s[0]);
+            s[1] = Ops::mma(kf[st % kKDepth][1].f, qf[st], s[1]);
             __builtin_amdgcn_sched_barrier(0);
         }
         // V^T operands of the first 16-key group travel while the softmax runs
@@ -320,7 +331,7 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const float p = (a.dbg & 4) ? s[sb][u * 8 + j] : __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
+                    const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
                     psum[j & 3] += p;
                     pf[sb][u][j] = static_cast<T>(p);
                 }
@@ -329,7 +340,6 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
         lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
         // ---- O^T += V^T . P^T : k slot (hh, j) of group g = 2*sb + u is key 16*g + 8*(j/4) + 4*hh + j%4 ----
         // accumulator row n' of o[mb] stands for LDS row 32*mb + n', i.e. dim 8 * (row % 16) + row / 16
-        if (!(a.dbg & 8))
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (g + 1 < 4) loadV(g + 1, (g + 1) & 1);
@@ -338,14 +348,18 @@ __global__ __launch_bounds__(kCtxThreads, 2) void ctxAttnMfma(T* __restrict__ ou
             for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        // the buffer of tile jt-1 (free since this iteration's barrier) takes tile jt+1, requested one iteration ago;
+        // the request for tile jt+2 follows and has a whole iteration to arrive
+        if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
+        if (jt + 2 < numKeyTiles) loadTile(jt + 2);
     }
 
     // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
     const float lTot = lRun + __shfl_xor(lRun, 32, kWave);
     const float inv = 1.0f / lTot;
-    __syncthreads();  // the K/V tiles are dead; reuse the storage as a [128][kLD] output tile
+    __syncthreads();  // the K/V tiles are dead; reuse the storage as a [BM][kLD] output tile
     T* sO = smem;
-    static_assert(kBM * kLD <= 2 * kStageElems, "the output tile must fit the staging storage");
+    static_assert(BM * kLD <= 2 * kStageElems, "the output tile must fit the staging storage");
 #pragma unroll
     for (int mb = 0; mb < kHD / 32; ++mb) {
 #pragma unroll
@@ -430,10 +444,10 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
     }
 }
 
-template <typename T>
+template <typename T, int NWV>
 diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
-    a.dbg = envInt("DIOPI_ROCM_CTX_DBG", 0);
-    a.tilesBound = static_cast<int>(ceilDiv(a.rows, kBM)) + a.batch;
+    constexpr int BM = NWV * 32;
+    a.tilesBound = static_cast<int>(ceilDiv(a.rows, BM)) + a.batch;
     const int64_t total = static_cast<int64_t>(a.tilesBound) * a.H;
     ROCM_CHECK(total < INT32_MAX / 2, "context attention: too many tiles for one launch");
     a.totalItems = static_cast<int>(total);
@@ -441,17 +455,17 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     void* planMem = nullptr;
     ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int2), &planMem));
     a.plan = static_cast<const int2*>(planMem);
-    const int maxTiles = static_cast<int>(ceilDiv(a.rows, kBM));
+    const int maxTiles = static_cast<int>(ceilDiv(a.rows, BM));
     const size_t planLds = (2 * static_cast<size_t>(a.batch) + maxTiles) * sizeof(int);
-    hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles);
+    hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles, BM);
     ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
     // exp(x) = exp2(x * log2(e)); the 1/sqrt(D) scaling of the scores is folded into the same factor
     const float scaleLog2 = static_cast<float>(1.4426950408889634 / std::sqrt(static_cast<double>(kHD)));
     constexpr int ldsBytes = 2 * kStageElems * static_cast<int>(sizeof(T));
-    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
     ROCM_HIP(granted);
-    hipLaunchKernelGGL(ctxAttnMfma<T>, dim3(grid), dim3(kCtxThreads), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
+    hipLaunchKernelGGL((ctxAttnMfma<T, NWV>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
                        static_cast<const T*>(v), a, scaleLog2);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
@@ -517,14 +531,18 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     const bool aligned =
         ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
     // the planning kernel keeps two ints per sequence and one per query tile in LDS
-    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBM + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
+    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
     const bool fast = D == kHD && aligned && planFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    // 256-row query tiles (8 waves share each K/V tile) once the sequences are long enough to fill them
+    const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
     switch (vQ.dtype) {
         case diopi_dtype_float16:
-            return fast ? launchMfma<half_t>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+            return fast ? (wide ? launchMfma<half_t, 8>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                                : launchMfma<half_t, 4>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
                         : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_bfloat16:
-            return fast ? launchMfma<bf16_t>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+            return fast ? (wide ? launchMfma<bf16_t, 8>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                                : launchMfma<bf16_t, 4>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
                         : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
         case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
