@@ -94,7 +94,7 @@ __device__ __forceinline__ float waveSumUniform(float v) {
     return (laneValue(v, 0) + laneValue(v, 16)) + (laneValue(v, 32) + laneValue(v, 48));
 }
 
-template <typename T, int GC>
+template <typename T, int GC, int HPW>
 __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
                                                                     SplitArgs sp) {
     using Ops = Mfma16<T>;
@@ -118,16 +118,23 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     const int tid = threadIdx.x;
     const int lane = tid % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    const int q = lane / 16;  // 16-lane group: tokens 8q .. 8q+7 of every 32-token step
-    const int c = lane % 16;  // 16-byte packet of the row segment; also the query head of the A operand
+    // HPW == 1: the wave streams one kv head; lane group q takes tokens 8q .. 8q+7 of every 32-token step.
+    // HPW == 4: the wave streams four adjacent kv heads (1 KiB contiguous per token, which the memory system likes
+    //           better); lane group q takes head q and the same 8 tokens per step as the other groups.  The four
+    //           heads share the products through a block-diagonal A operand: row m only carries probabilities in the
+    //           lane group of its own kv head, zeros elsewhere.
+    const int q = lane / 16;
+    const int c = lane % 16;  // 16-byte packet of the row segment; also the row (query head) of the A operand
     const int G = a.G;
-    const int hk = blockIdx.z * kRvWaves + wave;
+    const int R = HPW * G;    // query heads (rows of the A operand) of this wave, <= GC
+    const int hk = (blockIdx.z * kRvWaves + wave) * HPW;  // first kv head of the wave
     if (hk >= a.Hkv) return;
+    constexpr int kStep = HPW == 1 ? 32 : 8;  // tokens per step
     const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
     T* tile = &sP[wave][0];
     int32_t* slotW = &sSlotW[wave][0];
     float* statW = &sStat[wave][0];
-    const T* vHead = v + hk * kD + c * 8;
+    const T* vHead = v + (hk + (HPW == 1 ? 0 : q)) * kD + c * 8;
     const int64_t colBase = start + t0;
     const T* xBase = logits + static_cast<int64_t>(hk) * G * a.logitCols + colBase;
 
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
                 const int t = sub * kSub + 64 * k + lane;
                 const int64_t col = colBase + t;
                 xr[g][k] = -INFINITY;
-                if (g < G && t < nTokR && col >= 0 && col < a.logitCols) xr[g][k] = static_cast<float>(xBase[static_cast<int64_t>(g) * a.logitCols + t]);
+                if (g < R && t < nTokR && col >= 0 && col < a.logitCols) xr[g][k] = static_cast<float>(xBase[static_cast<int64_t>(g) * a.logitCols + t]);
             }
         }
     };
@@ -165,8 +172,9 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     u32x4 rowsV[8];
     auto issueV = [&](int step) {
         int32_t sidx[8];
-        *reinterpret_cast<u32x4*>(&sidx[0]) = *reinterpret_cast<const u32x4*>(slotW + 32 * step + 8 * q);
-        *reinterpret_cast<u32x4*>(&sidx[4]) = *reinterpret_cast<const u32x4*>(slotW + 32 * step + 8 * q + 4);
+        const int first = HPW == 1 ? 32 * step + 8 * q : 8 * step;
+        *reinterpret_cast<u32x4*>(&sidx[0]) = *reinterpret_cast<const u32x4*>(slotW + first);
+        *reinterpret_cast<u32x4*>(&sidx[4]) = *reinterpret_cast<const u32x4*>(slotW + first + 4);
 #pragma unroll
         for (int r = 0; r < 8; ++r) rowsV[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(sidx[r]) * rowStride));
     };
@@ -188,13 +196,13 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
 
     for (int sub = 0; sub < nSub; ++sub) {
         const int nTok = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
-        const int nSteps = (nTok + 31) / 32;
+        const int nSteps = (nTok + kStep - 1) / kStep;
         // ---- softmax of the sub-tile ----
         waveLdsFence();
         bool moved = false;
 #pragma unroll
         for (int g = 0; g < GC; ++g) {
-            if (g < G) {
+            if (g < R) {
                 const float mNew = fmaxf(mRun[g], waveMaxUniform(fmaxf(xr[g][0], xr[g][1])));
                 const float mUse = (mNew == -INFINITY) ? 0.f : mNew;  // a head whose logits are all -inf keeps p = 0
                 const float p0 = __expf(xr[g][0] - mUse);
@@ -219,14 +227,16 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
             for (int e = 0; e < 8; ++e) acc[e] *= al;
         }
         // ---- P . V on the matrix cores ----
-        const T* pRow = tile + (c < G ? c : 0) * kTilePitch + 8 * q;
+        // A operand: row c, the 8 tokens of this lane group's k slots; rows of other kv heads contribute zeros
+        const bool rowLive = HPW == 1 ? c < G : (c < R && c / G == q);
+        const T* pRow = tile + (c < R ? c : 0) * kTilePitch + (HPW == 1 ? 8 * q : 0);
         for (int s = 0; s < nSteps; ++s) {
             union {
                 u32x4 u;
                 Frag f;
             } pa;
-            pa.u = *reinterpret_cast<const u32x4*>(pRow + 32 * s);
-            if (c >= G) pa.u = u32x4{0u, 0u, 0u, 0u};
+            pa.u = *reinterpret_cast<const u32x4*>(pRow + kStep * s);
+            if (!rowLive) pa.u = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 union {
@@ -261,7 +271,7 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     waveLdsFence();
     const bool single = L <= sp.TT;  // the whole sequence lives in this range
     const int64_t split = blockIdx.y;
-    if (!single && lane < G) {
+    if (!single && lane < R) {
         // lane g publishes (max, denominator) of query head g
         float mg = -INFINITY;
 #pragma unroll
@@ -273,7 +283,7 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int g = 4 * q + r;
-        if (g >= G) continue;
+        if (g >= R) continue;
         const int qh = hk * G + g;
         if (single) {
             const float inv = 1.f / statW[g];
@@ -415,20 +425,32 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
         sp.partMl = reinterpret_cast<float*>(static_cast<char*>(scratch) + accBytes);
     }
     ROCM_CHECK(sp.splits <= 65535, "max_input_len %d needs more than 65535 ranges of %d tokens", a.maxInputLen, TT);
-    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits), static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves)));
-#define ROCM_RVW_CASE(GC)                                                                                                                   \
-    hipLaunchKernelGGL((softmaxReduceVWave<T, GC>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
+    // four adjacent kv heads per wave (1 KiB contiguous per token) when their query heads fit the 16 rows of a product
+    const bool quad = a.G <= 4 && a.Hkv % 4 == 0 && envInt("DIOPI_ROCM_REDUCEV_QUAD", 1) != 0;
+    const int hpw = quad ? 4 : 1;
+    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits), static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves * hpw)));
+#define ROCM_RVW_CASE(GC, HPW)                                                                                                                   \
+    hipLaunchKernelGGL((softmaxReduceVWave<T, GC, HPW>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
                        static_cast<const T*>(v), a, sp)
-    if (a.G <= 1) {
-        ROCM_RVW_CASE(1);
-    } else if (a.G <= 2) {
-        ROCM_RVW_CASE(2);
-    } else if (a.G <= 4) {
-        ROCM_RVW_CASE(4);
-    } else if (a.G <= 8) {
-        ROCM_RVW_CASE(8);
+    const int rows = hpw * a.G;
+    if (quad) {
+        if (rows <= 4) {
+            ROCM_RVW_CASE(4, 4);
+        } else if (rows <= 8) {
+            ROCM_RVW_CASE(8, 4);
+        } else {
+            ROCM_RVW_CASE(16, 4);
+        }
+    } else if (rows <= 1) {
+        ROCM_RVW_CASE(1, 1);
+    } else if (rows <= 2) {
+        ROCM_RVW_CASE(2, 1);
+    } else if (rows <= 4) {
+        ROCM_RVW_CASE(4, 1);
+    } else if (rows <= 8) {
+        ROCM_RVW_CASE(8, 1);
     } else {
-        ROCM_RVW_CASE(16);
+        ROCM_RVW_CASE(16, 1);
     }
 #undef ROCM_RVW_CASE
     ROCM_LAUNCH_CHECK();
