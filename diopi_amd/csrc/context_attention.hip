@@ -238,9 +238,41 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
             }
         }
     };
+    // The same staging work cut into pieces of one or two instructions each, so that it can be dealt out between the
+    // matrix instructions of the second product: first the LDS writes of tile jt+1 (registers requested one iteration
+    // ago), then the global requests of tile jt+2 into the same registers.  Unconditional: rows are clamped and a
+    // surplus tile lands in a buffer nobody reads any more.
+    constexpr int kPiecesVW = 8 * kVItems, kPiecesKW = kKPasses, kPiecesKL = kKPasses, kPiecesVL = 2 * kVItems;
+    constexpr int kPieces = kPiecesVW + kPiecesKW + kPiecesKL + kPiecesVL;
+    auto stagePiece = [&](int idx, int jt) {
+        T* sKn = smem + ((jt + 1) & 1) * kStageElems;
+        if (idx < kPiecesVW) {
+            const int it = idx / 8, e = idx % 8;
+            const int ci = wave * kVItems + it;
+            const int posd = 8 * (ci / 2) + 4 * (ci % 2) + q4;
+            uint32_t* sVt32 = reinterpret_cast<uint32_t*>(sKn + kBN * kLD);
+            sVt32[(16 * e + ldC) * (kVP / 2) + posd] =
+                __builtin_amdgcn_perm(vReg[it][1][e / 2], vReg[it][0][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
+        } else if (idx < kPiecesVW + kPiecesKW) {
+            const int it = idx - kPiecesVW;
+            *reinterpret_cast<u32x4*>(sKn + (ldR + it * kRowsPerPass) * kLD + ldC * 8) = kReg[it];
+        } else if (idx < kPiecesVW + kPiecesKW + kPiecesKL) {
+            const int it = idx - kPiecesVW - kPiecesKW;
+            int row = (jt + 2) * kBN + ldR + it * kRowsPerPass;
+            row = row < L ? row : L - 1;
+            kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
+        } else if (idx < kPieces) {
+            const int k2 = idx - kPiecesVW - kPiecesKW - kPiecesKL;
+            const int it = k2 / 2, h2 = k2 % 2;
+            const int ci = wave * kVItems + it;
+            int row = (jt + 2) * kBN + 16 * (ci / 2) + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * (ci % 2) + h2;
+            row = row < L ? row : L - 1;
+            vReg[it][h2] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
+        }
+    };
     loadTile(0);
     stageTile(0);
-    if (numKeyTiles > 1) loadTile(1);
+    loadTile(1);
 
     for (int jt = 0; jt < numKeyTiles; ++jt) {
         // One barrier per tile: tile jt is staged and every wave has left tile jt-1, whose buffer now takes tile
@@ -252,8 +284,8 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         const int key0 = jt * kBN;
         if (key0 > waveRowHi) {
             // entirely above the diagonal for this wave: only the staging duty remains
-            if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
-            if (jt + 2 < numKeyTiles) loadTile(jt + 2);
+#pragma unroll
+            for (int idx = 0; idx < kPieces; ++idx) stagePiece(idx, jt);
             continue;
         }  // entirely above the diagonal for this wave (barriers are at the loop top)
 
@@ -345,13 +377,16 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
             if (g + 1 < 4) loadV(g + 1, (g + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int mb = 0; mb < kHD / 32; ++mb) {
+                o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
+                // staging pieces ride in the shadow of the matrix instruction just issued (the buffer of tile jt-1
+                // is free since this iteration's barrier)
+                constexpr int kPerSlot = (kPieces + 15) / 16;
+#pragma unroll
+                for (int k2 = 0; k2 < kPerSlot; ++k2) stagePiece((g * 4 + mb) * kPerSlot + k2, jt);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        // the buffer of tile jt-1 (free since this iteration's barrier) takes tile jt+1, requested one iteration ago;
-        // the request for tile jt+2 follows and has a whole iteration to arrive
-        if (jt + 1 < numKeyTiles) stageTile((jt + 1) & 1);
-        if (jt + 2 < numKeyTiles) loadTile(jt + 2);
     }
 
     // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
