@@ -132,7 +132,9 @@ __global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ p
 
 template <typename T, int NWV>
 __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-                                                               CtxArgs a, float scaleLog2) {
+                                                               CtxArgs a) {
+    // exp(x / sqrt(D)) = exp2(x * log2(e) / sqrt(D)): one literal factor
+    constexpr float scaleLog2 = 0.12751743082459868f;  // log2(e) / sqrt(128)
     using Ops = Mfma32<T>;
     using Frag = typename Ops::Frag;
     constexpr int BM = NWV * 32;  // query rows per work-group: each of the NWV waves owns 32 of them
@@ -394,6 +396,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     const float inv = 1.0f / lTot;
     __syncthreads();  // the K/V tiles are dead; reuse the storage as a [BM][kLD] output tile
     T* sO = smem;
+    static_assert(kHD == 128, "scaleLog2 is written out for head size 128");
     static_assert(BM * kLD <= 2 * kStageElems, "the output tile must fit the staging storage");
 #pragma unroll
     for (int mb = 0; mb < kHD / 32; ++mb) {
@@ -495,13 +498,11 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles, BM);
     ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
-    // exp(x) = exp2(x * log2(e)); the 1/sqrt(D) scaling of the scores is folded into the same factor
-    const float scaleLog2 = static_cast<float>(1.4426950408889634 / std::sqrt(static_cast<double>(kHD)));
     constexpr int ldsBytes = 2 * kStageElems * static_cast<int>(sizeof(T));
     static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
     ROCM_HIP(granted);
     hipLaunchKernelGGL((ctxAttnMfma<T, NWV>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), a, scaleLog2);
+                       static_cast<const T*>(v), a);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
