@@ -29,6 +29,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0    # dense fp16 / bf16
 WARM_SECONDS = 0.3          # untimed load before every timed region (clock ramp)
+# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one counter per run, commands
+# and raw readings in profiles/all_operators_cfg1-5_hbm_traffic.txt) for the seeded cfg3 workload, each counter scaled
+# by what it reads for a plain copy of known size (the 65536-row DestIndexCopyKV sweep: 1.9854 KiB per FETCH_SIZE
+# count, 1.0000 KiB per WRITE_SIZE count).  The counters cannot be read from inside this script.
+MEASURED_TRAFFIC_CFG3 = {
+    "tokenAttStaged": int((314577.1 * 1.9854 + 5569.2) * 1024),
+    "softmaxReduceVWave+Merge": int(((315472.4 + 1684.0) * 1.9854 + 2973.8 + 512.0) * 1024),
+}
 
 
 def main():
@@ -38,6 +46,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -74,7 +83,7 @@ def main():
         # until that much time has passed, so that the K timed steps do not include the ramp
         t_warm = time.perf_counter()
         i = warmup
-        while time.perf_counter() - t_warm < WARM_SECONDS:
+        while time.perf_counter() - t_warm < args.warm_seconds:
             for _ in range(8):
                 step_fn(i)
                 i += 1
@@ -336,9 +345,10 @@ def main():
             kname, kms, kbytes = "tokenAttStaged (diopiTokenAttentionInference)", head["ms_att"], head["b_att"]
         else:
             kname, kms, kbytes = "softmaxReduceVWave+Merge (diopiTokenSoftmaxReduceVInference)", head["ms_red"], head["b_red"]
+        traffic = MEASURED_TRAFFIC_CFG3.get(kname.split(" ")[0]) if head["total"] == 78106 else None
         ach = kbytes / (kms * 1e-3) / 1e9
         line["roofline"] = {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}
+                            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}
         if head["cpu"] is not None:
             c = head["cpu"]
             line["cpu_baseline"] = {"value": c["tokens_per_s"], "unit": "tokens/s", "cores": c["cores"], "kind": "port", "sample": c["sample"]}
