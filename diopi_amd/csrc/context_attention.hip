@@ -126,7 +126,11 @@ __global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ p
     for (int s = 0; s < a.batch; ++s) {
         const int nt = sTiles[s];
         const int rank = nt > 0 ? sTiles[a.batch + s] : 0;
-        for (int t = tid; t < nt; t += kPlanThreads) plan[sTiles[2 * a.batch + t] + rank] = make_int2(s, t);
+        for (int t = tid; t < nt; t += kPlanThreads) {
+            // overlapping sequences (a caller error) could count more tiles than the bound the table is sized for
+            const int pos = (t < maxTiles ? sTiles[2 * a.batch + t] : a.tilesBound) + rank;
+            if (pos < a.tilesBound) plan[pos] = make_int2(s, t);
+        }
     }
 }
 

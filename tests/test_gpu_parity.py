@@ -454,6 +454,30 @@ def test_context_attention_ragged_lengths():
                           f"ragged {dt} {idt}")
 
 
+def test_context_attention_many_short_sequences():
+    # more sequences than lanes in a wave or threads in the planning group's first pass, empty ones included
+    rng = np.random.Generator(np.random.PCG64(77))
+    lens = rng.integers(0, 40, size=1100).tolist()
+    lens[5], lens[700] = 300, 129
+    starts = np.concatenate(([0], np.cumsum(lens)[:-1])).tolist()
+    T = int(sum(lens))
+    g = gen(602)
+    q, k, v = ((torch.randn(T, 2, 128, generator=g) * 0.5).to(torch.float16).to(DEV) for _ in range(3))
+    _context_case(q, k, v, torch.tensor(starts, dtype=torch.int32, device=DEV), torch.tensor(lens, dtype=torch.int32, device=DEV), max(lens),
+                  torch.float16, "1100 short sequences")
+
+
+def test_context_attention_long_odd_lengths_whole_output():
+    # long enough for the 256-row query tiles; lengths that are no multiple of any tile size; every row checked
+    lens = [1531, 1099]
+    starts = [0, 1531]
+    g = gen(603)
+    for dt in (torch.float16, torch.bfloat16):
+        q, k, v = ((torch.randn(sum(lens), 2, 128, generator=g) * 0.5).to(dt).to(DEV) for _ in range(3))
+        _context_case(q, k, v, torch.tensor(starts, dtype=torch.int32, device=DEV), torch.tensor(lens, dtype=torch.int32, device=DEV), max(lens), dt,
+                      f"two long sequences {dt}")
+
+
 def test_context_attention_config4_scaled():
     w = W.cfg4(DEV, seed=4, scale=0.125)  # 8 sequences of 128..512 tokens
     _context_case(w["q"], w["k"], w["v"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], torch.float16, "cfg4 x 1/8")
