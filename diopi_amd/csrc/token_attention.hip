@@ -84,13 +84,14 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttMfma(T* __restrict__ out,
     using Ops = MfmaOps<T>;
     using Frag = typename Ops::Frag;
     constexpr int kGroups = TT / kTokGroup;
-    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
-    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
-    // sparsely populated late tiles
-    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
+    // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
+    // time), y over sequences, z over token tiles, with the sequence rotated by the tile index so that consecutive
+    // work-groups (which the dispatcher deals round-robin to the 8 XCDs) mix tiles of different sequences: with
+    // ragged lengths no XCD is left with only the sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * TT;
     if (t0 >= L) return;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int lane = threadIdx.x % kWave;
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttMfma(T* __restrict__ out,
         slotOff[g] = slot * rowStride;
     }
 
-    const int hkBegin = blockIdx.z * HB;
+    const int hkBegin = blockIdx.x * HB;
     const int hkEnd = (hkBegin + HB < a.Hkv) ? hkBegin + HB : a.Hkv;
     for (int hk = hkBegin + wave; hk < hkEnd; hk += kAttWaves) {
         // A fragments: row n is query head hk*G + n (zero beyond the group)
@@ -185,13 +186,14 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     __shared__ __attribute__((aligned(16))) T stage[kAttWaves][16 * kStagePitch];
     __shared__ int sSlot[1024];   // slot index of every token of the tile (TT <= 1024)
 
-    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
-    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
-    // sparsely populated late tiles
-    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
+    // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
+    // time), y over sequences, z over token tiles, with the sequence rotated by the tile index so that consecutive
+    // work-groups (which the dispatcher deals round-robin to the 8 XCDs) mix tiles of different sequences: with
+    // ragged lengths no XCD is left with only the sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * TT;
     if (t0 >= L) return;
     const int nTok = static_cast<int>((L - t0 < TT) ? L - t0 : TT);
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
@@ -211,7 +213,7 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     const int TPH = kAttWaves / HS;
     const int hs = wave % HS;
     const int tph = wave / HS;
-    const int hk0 = (blockIdx.z * HS + hs) * HW;
+    const int hk0 = (blockIdx.x * HS + hs) * HW;
     if (hk0 >= a.Hkv) return;
     const int64_t rowStride = static_cast<int64_t>(a.Hkv) * D;
     T* myStage = stage[wave];
@@ -278,13 +280,14 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
 template <typename T, typename AccT>
 __global__ __launch_bounds__(kAttThreads) void tokenAttGeneric(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, DecodeArgs a, int TT,
                                                                AccT scale) {
-    // x runs over sequences, y over token tiles, rotated so that consecutive work-groups (which the dispatcher deals
-    // round-robin to the 8 XCDs) mix tiles of different sequences: with ragged lengths no XCD is left with only the
-    // sparsely populated late tiles
-    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
+    // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
+    // time), y over sequences, z over token tiles, with the sequence rotated by the tile index so that consecutive
+    // work-groups (which the dispatcher deals round-robin to the 8 XCDs) mix tiles of different sequences: with
+    // ragged lengths no XCD is left with only the sparsely populated late tiles
+    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * TT;
     if (t0 >= L) return;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L);
@@ -314,7 +317,7 @@ diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void
     // kv heads per work-group: about 256 KiB of K per group, at least one head per wave
     int HB = a.Hkv < 8 ? a.Hkv : 8;
     HB = envInt("DIOPI_ROCM_TOKATT_HB", HB);
-    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(ceilDiv(a.Hkv, HB)));
+    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HB)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
     if (a.D == 128) {
         hipLaunchKernelGGL((tokenAttMfma<T, 4, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
                            static_cast<const T*>(k), a, HB, scale);
@@ -328,17 +331,21 @@ diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void
 
 template <typename T>
 diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a, float scale) {
-    // heads per wave, head slots per work-group (waves beyond the head slots take other token units)
-    const int HW = a.Hkv >= 16 ? 4 : (a.Hkv >= 8 ? 2 : 1);
+    // heads per wave, head slots per work-group (waves beyond the head slots take other token units).  One head per
+    // wave and short token tiles measured best once the head groups of a tile are dispatched next to each other:
+    // neighbouring work-groups then stream neighbouring pieces of the same cache rows at the same time.
+    int HW = 1;
+    HW = envInt("DIOPI_ROCM_TOKATT_HW", HW);
+    if (HW != 1 && HW != 2 && HW != 4) HW = 1;
     const int slots = static_cast<int>(ceilDiv(a.Hkv, HW));
-    const int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
-    // tokens per work-group: about half a MiB of K per group
-    int TT = static_cast<int>((512 * 1024) / (static_cast<int64_t>(HS) * HW * 128 * sizeof(T)));
-    TT = envInt("DIOPI_ROCM_TOKATT_TT", TT);
+    int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
+    HS = envInt("DIOPI_ROCM_TOKATT_HS", HS);
+    if (HS != 1 && HS != 2 && HS != 4) HS = 1;
+    int TT = envInt("DIOPI_ROCM_TOKATT_TT", 128);  // tokens per work-group
     TT = TT / 64 * 64;
     if (TT < 64) TT = 64;
     if (TT > 1024) TT = 1024;
-    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)));
+    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
 #define ROCM_STAGED_CASE(HWC)                                                                                                                         \
     hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),                  \
                        static_cast<const T*>(k), a, TT, HS, scale)
@@ -357,7 +364,7 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
 template <typename T, typename AccT>
 diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a) {
     const int TT = 64;
-    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
+    const dim3 grid(1, static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
     const AccT scale = static_cast<AccT>(1.0 / std::sqrt(static_cast<double>(a.D)));
     hipLaunchKernelGGL((tokenAttGeneric<T, AccT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
                        static_cast<const T*>(k), a, TT, scale);

@@ -103,12 +103,14 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     __shared__ __attribute__((aligned(16))) int32_t sSlotW[kRvWaves][kSub];
     __shared__ __attribute__((aligned(16))) float sStat[kRvWaves][16];
 
-    // x runs over sequences, y over token ranges, rotated so that consecutive work-groups (dealt round-robin to the 8
-    // XCDs) mix ranges of different sequences: with ragged lengths no XCD is left with only the sparse late ranges
-    const int i = static_cast<int>((blockIdx.x + blockIdx.y) % gridDim.x);
+    // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
+    // time), y over sequences, z over token ranges, with the sequence rotated by the range index so that consecutive
+    // work-groups (dealt round-robin to the 8 XCDs) mix ranges of different sequences: with ragged lengths no XCD is
+    // left with only the sparse late ranges
+    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.y) * sp.TT;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * sp.TT;
     if (t0 >= L) return;
     const int64_t tEnd = (t0 + sp.TT < L) ? t0 + sp.TT : L;
     const int nTokR = static_cast<int>(tEnd - t0);
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     const int c = lane % 16;  // 16-byte packet of the row segment; also the row (query head) of the A operand
     const int G = a.G;
     const int R = HPW * G;    // query heads (rows of the A operand) of this wave, <= GC
-    const int hk = (blockIdx.z * kRvWaves + wave) * HPW;  // first kv head of the wave
+    const int hk = (blockIdx.x * kRvWaves + wave) * HPW;  // first kv head of the wave
     if (hk >= a.Hkv) return;
     constexpr int kStep = HPW == 1 ? 32 : 8;  // tokens per step
     const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     }
     waveLdsFence();
     const bool single = L <= sp.TT;  // the whole sequence lives in this range
-    const int64_t split = blockIdx.y;
+    const int64_t split = blockIdx.z;
     if (!single && lane < R) {
         // lane g publishes (max, denominator) of query head g
         float mg = -INFINITY;
@@ -424,11 +426,12 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
         sp.partAcc = static_cast<float*>(scratch);
         sp.partMl = reinterpret_cast<float*>(static_cast<char*>(scratch) + accBytes);
     }
+    ROCM_CHECK(a.batch <= 65535, "batch %d exceeds the launch limit of 65535 sequences", a.batch);
     ROCM_CHECK(sp.splits <= 65535, "max_input_len %d needs more than 65535 ranges of %d tokens", a.maxInputLen, TT);
     // four adjacent kv heads per wave (1 KiB contiguous per token) when their query heads fit the 16 rows of a product
-    const bool quad = a.G <= 4 && a.Hkv % 4 == 0 && envInt("DIOPI_ROCM_REDUCEV_QUAD", 1) != 0;
+    const bool quad = a.G <= 4 && a.Hkv % 4 == 0 && envInt("DIOPI_ROCM_REDUCEV_QUAD", 0) != 0;
     const int hpw = quad ? 4 : 1;
-    const dim3 grid(static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits), static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves * hpw)));
+    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves * hpw)), static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits));
 #define ROCM_RVW_CASE(GC, HPW)                                                                                                                   \
     hipLaunchKernelGGL((softmaxReduceVWave<T, GC, HPW>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
                        static_cast<const T*>(v), a, sp)
