@@ -180,7 +180,10 @@ def main():
             s["inv"] = torch.empty(T, dtype=torch.float32, device=dev)
             s["qo"] = torch.empty_like(s["q"])
             s["ko"] = torch.empty_like(s["k"])
-            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "out", "inv", "q", "k", "cos", "sin", "qo", "ko")})
+            # full-width tables for the fused in-place operator (same angles in both halves)
+            s["cos2"] = torch.cat((s["cos"], s["cos"]), -1).contiguous()
+            s["sin2"] = torch.cat((s["sin"], s["sin"]), -1).contiguous()
+            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "out", "inv", "q", "k", "cos", "sin", "qo", "ko", "cos2", "sin2")})
 
         def norm(i):
             h = hs[i % 3]
@@ -191,8 +194,14 @@ def main():
             check(impl.diopiRotaryEmbedding(ctx.handle, h["qo"].handle, h["q"].handle, h["cos"].handle, h["sin"].handle, False, False), "diopiRotaryEmbedding")
             check(impl.diopiRotaryEmbedding(ctx.handle, h["ko"].handle, h["k"].handle, h["cos"].handle, h["sin"].handle, False, False), "diopiRotaryEmbedding")
 
+        def rot2(i):
+            # in place: the buffers keep rotating by the same angles, which does not change the work
+            h = hs[i % 3]
+            check(impl.diopiRotaryEmbeddingV2(ctx.handle, h["qo"].handle, h["ko"].handle, h["cos2"].handle, h["sin2"].handle, D), "diopiRotaryEmbeddingV2")
+
         ms_n = timed(norm)
         ms_r = timed(rot)
+        ms_r2 = timed(rot2)
         cpu_n = cpu_r = None
         if not args.no_cpu:
             xc, wc = sets[0]["x"].cpu(), sets[0]["weight"].cpu()
@@ -203,6 +212,8 @@ def main():
             cpu_r = dict(seconds=round(2 * t, 4), GBs=round(W.rotary_bytes(T, H, D, 2) / t / 1e9, 2), cores=cores, sample="q call timed, k call assumed equal")
         record("diopiRMSNorm", "cfg2 bf16 [16384,4096]", ms_n, W.rmsnorm_fwd_bytes(T, n2, 2), "hbm", "bf16", cpu_n)
         record("diopiRotaryEmbedding x2 (q,k)", "cfg2 bf16 [16384,32,128]", ms_r, 2 * W.rotary_bytes(T, H, D, 2), "hbm", "bf16", cpu_r)
+        record("diopiRotaryEmbeddingV2 (q,k in place, one launch)", "cfg2 bf16 [16384,32,128] x2", ms_r2, 2 * 2 * T * H * D * 2 + 2 * T * D * 2, "hbm", "bf16",
+               None, note="widening beyond the seven hot-path operators; bytes = read+write of q and k, full-width cos/sin once")
         del sets, hs
         torch.cuda.empty_cache()
 

@@ -317,6 +317,7 @@ diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void
     // kv heads per work-group: about 256 KiB of K per group, at least one head per wave
     int HB = a.Hkv < 8 ? a.Hkv : 8;
     HB = envInt("DIOPI_ROCM_TOKATT_HB", HB);
+    ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
     const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HB)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
     if (a.D == 128) {
         hipLaunchKernelGGL((tokenAttMfma<T, 4, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
@@ -345,6 +346,7 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     TT = TT / 64 * 64;
     if (TT < 64) TT = 64;
     if (TT > 1024) TT = 1024;
+    ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
     const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
 #define ROCM_STAGED_CASE(HWC)                                                                                                                         \
     hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),                  \
@@ -364,6 +366,7 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
 template <typename T, typename AccT>
 diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a) {
     const int TT = 64;
+    ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
     const dim3 grid(1, static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
     const AccT scale = static_cast<AccT>(1.0 / std::sqrt(static_cast<double>(a.D)));
     hipLaunchKernelGGL((tokenAttGeneric<T, AccT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),

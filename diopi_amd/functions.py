@@ -66,6 +66,16 @@ def rotary_emb(input: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, conj: 
     return out
 
 
+def rotary_emb_v2(query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, dim: int, ctx: Optional[rt.Context] = None):
+    """In place on query and key, like the reference wrapper (diopi_functions.py:8051-8056)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, query):
+        keep, h = _handles(query, key, cos, sin)
+        ret = rt.libs().impl.diopiRotaryEmbeddingV2(ctx.handle, *h, int(dim))
+    check_returncode(ret, "diopiRotaryEmbeddingV2")
+    return query, key
+
+
 def rms_norm(input: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
              ctx: Optional[rt.Context] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     ctx = _ctx(ctx)

@@ -135,6 +135,7 @@ class _Libs:
             getattr(impl, name).argtypes = []
         b = ctypes.c_bool
         impl.diopiRotaryEmbedding.argtypes = [vp, vp, vp, vp, vp, b, b]
+        impl.diopiRotaryEmbeddingV2.argtypes = [vp, vp, vp, vp, vp, i64]
         impl.diopiRMSNorm.argtypes = [vp, vp, vp, vp, _SizeStruct, vp, vp, ctypes.c_double]
         impl.diopiRMSNormBackward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, _SizeStruct, ctypes.c_double]
         impl.diopiDestIndexCopyKV.argtypes = [vp, vp, vp, vp]
@@ -148,6 +149,7 @@ class _Libs:
 # Every symbol include/diopi/functions.h and include/diopi/functions_ext.h declare.
 OPERATOR_SYMBOLS = (
     "diopiRotaryEmbedding",
+    "diopiRotaryEmbeddingV2",
     "diopiRMSNorm",
     "diopiRMSNormBackward",
     "diopiDestIndexCopyKV",

@@ -39,6 +39,18 @@ DIOPI_API diopiError_t diopiRotaryEmbedding(diopiContextHandle_t ctx, diopiTenso
                                             diopiConstTensorHandle_t sin, const bool conj, const bool interleaved);
 
 /*
+ * Rotary position embedding of query and key, in place, with full-width tables (the lightllm form).
+ * reference: functions_ext.h:649-650 (statement: customized_test.py:843-852).
+ *   query [T, Hq*dim] and key [T, Hk*dim] are viewed as [T, heads, dim]; cos, sin hold T*dim elements ([T, 1, dim]).
+ *   x[.., d]         <- x[.., d]*cos[d]             - x[.., d + dim/2]*sin[d]              (d < dim/2)
+ *   x[.., d + dim/2] <- x[.., d + dim/2]*cos[d + dim/2] + x[.., d]*sin[d + dim/2]
+ * Arithmetic is fp32 (fp64 for fp64 tensors) with one rounding to the element type.
+ * dtypes: float16, bfloat16, float32, float64 (query, key, cos, sin share one dtype).
+ */
+DIOPI_API diopiError_t diopiRotaryEmbeddingV2(diopiContextHandle_t ctx, diopiTensorHandle_t query, diopiTensorHandle_t key, diopiConstTensorHandle_t cos,
+                                              diopiConstTensorHandle_t sin, int64_t dim);
+
+/*
  * RMS normalisation over the trailing `normalized_shape` dimensions.
  * reference: functions_ext.h:45-46.
  *   inv_rms[row] = rsqrt(mean(x[row]^2) + eps)         (fp32 accumulate; fp64 for fp64 input)

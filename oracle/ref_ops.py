@@ -1,4 +1,5 @@
-"""CPU oracle for the seven LLaMA-inference operators.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the LLaMA-inference operators (the seven of the hot path and
+diopiRotaryEmbeddingV2).  TEST INFRASTRUCTURE ONLY.
 
 This module restates, on the CPU with plain ATen (torch) and numpy calls, what the reference
 computes for each operator.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
@@ -13,6 +14,8 @@ rms_norm                     impl/torch/functions/functions_ext.cpp:66-80,
 rms_norm_backward            functions_ext.cpp:82-107, layer_norm_cuda_kernel.cu:402, 444, 572-717
 rotary_emb                   functions_ext.cpp:43-64, functions_ext/rotary.cu:26-44;
                              customized_test.py:374-390
+rotary_emb_v2                customized_test.py:843-852 (the torch implementation has no body for
+                             diopiRotaryEmbeddingV2; declaration functions_ext.h:649-650)
 destindex_copy_kv            functions_lightllm.cpp:18-26; customized_test.py:694-696
 token_attention              functions_lightllm.cpp:53-80; customized_test.py:698-713
 token_softmax_reducev        functions_lightllm.cpp:82-107; customized_test.py:715-733
@@ -39,6 +42,10 @@ How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"
   rotary_emb           position 0 is the identity bit for bit, norm preservation per pair,
                        conj undoes the rotation, the reference's broadcasting shapes
                        (diopi_configs.py:9066-9074), empty tensors (9093)
+  rotary_emb_v2        tables of ones and zeros are the identity bit for bit, duplicated table halves
+                       reproduce rotary_emb on the [T, heads, dim] view, explicit Python loops in
+                       float64 with tables whose halves differ, the reference's case shape
+                       (diopi_configs.py:9107-9135)
   destindex_copy_kv    the reference fixtures dest_loc=(0..4),(14..17) into 120 rows
                        (diopi_configs.py:9321-9333), untouched rows compared byte for byte
   token_attention      the reference's integer fixture (diopi_configs.py:9541-9558) read against an
@@ -132,6 +139,20 @@ def rotary_emb(input: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, conj: 
         o2 = -x1 * s + x2 * c
     out = torch.cat((o1, o2), dim=-1)
     return out if exact else out.to(input.dtype)
+
+
+def rotary_emb_v2(query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, dim: int, exact: bool = False):
+    """customized_test.py:843-852: x * cos + rotate_half(x) * sin on the [T, heads, dim] views of query and key, every
+    product and the sum in the tensor dtype (float64 when exact).  Returns new tensors with the input shapes."""
+    def one(x: torch.Tensor) -> torch.Tensor:
+        xv = x.reshape(x.shape[0], -1, dim)
+        c, s = cos.reshape(cos.shape[0], 1, dim), sin.reshape(sin.shape[0], 1, dim)
+        if exact:
+            xv, c, s = xv.to(torch.float64), c.to(torch.float64), s.to(torch.float64)
+        x1, x2 = xv.chunk(2, dim=-1)
+        rotated = torch.cat((-x2, x1), dim=-1)
+        return (xv * c + rotated * s).reshape(x.shape)
+    return one(query), one(key)
 
 
 def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

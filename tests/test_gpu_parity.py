@@ -261,6 +261,61 @@ def test_rotary_config2_full_size():
         assert same > 0.999
 
 
+def _rotary_v2_case(T, Hq, Hk, dim, dt, what, true_rotation=True):
+    g = gen(700 + T)
+    q = torch.randn(T, Hq * dim, generator=g).to(dt).to(DEV)
+    k = torch.randn(T, Hk * dim, generator=g).to(dt).to(DEV)
+    if true_rotation:
+        ang = torch.rand(T, 1, dim // 2, generator=g) * 6.28
+        cos, sin = torch.cat((ang.cos(), ang.cos()), -1).to(dt).to(DEV), torch.cat((ang.sin(), ang.sin()), -1).to(dt).to(DEV)
+    else:
+        cos, sin = torch.randn(T, 1, dim, generator=g).to(dt).to(DEV), torch.randn(T, 1, dim, generator=g).to(dt).to(DEV)
+    q0, k0 = q.clone(), k.clone()
+    before = snapshot(cos, sin)
+    F.rotary_emb_v2(q, k, cos, sin, dim)
+    assert_unmodified(before, cos, sin)
+    rq, rk = O.rotary_emb_v2(q0.cpu(), k0.cpu(), cos.cpu(), sin.cpu(), dim)
+    eq, ek = O.rotary_emb_v2(q0.cpu(), k0.cpu(), cos.cpu(), sin.cpu(), dim, exact=True)
+    tol = TOL[dt]
+    for got, ref, ex, name in ((q, rq, eq, "query"), (k, rk, ek, "key")):
+        assert_close(got.cpu(), ref, what=f"{what} {name} vs reference composition", **tol)
+        assert_close(got.cpu(), ex, what=f"{what} {name} vs float64", **tol)
+    say(what, "query max_abs/rel vs f64: %.3e %.3e" % report(q.cpu(), eq))
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_rotary_v2_reference_case_and_variants(dtype):
+    dt = TORCH_DTYPES[dtype]
+    _rotary_v2_case(8, 32, 32, 128, dt, f"rotary v2 reference case (8, 4096) {dtype}")  # diopi_configs.py:9107-9135
+    _rotary_v2_case(5, 8, 2, 64, dt, f"rotary v2 grouped heads {dtype}")
+    _rotary_v2_case(3, 3, 1, 12, dt, f"rotary v2 odd sizes (element-wise kernel) {dtype}", true_rotation=False)
+    _rotary_v2_case(4, 5, 3, 128, dt, f"rotary v2 unrelated table halves {dtype}", true_rotation=False)
+
+
+def test_rotary_v2_matches_two_rotary_calls_at_config2_size():
+    w = W.cfg2(DEV, seed=2)
+    T, H, D = w["T"], w["H"], w["D"]
+    cos, sin = torch.cat((w["cos"], w["cos"]), -1).contiguous(), torch.cat((w["sin"], w["sin"]), -1).contiguous()
+    q, k = w["q"].reshape(T, H * D).clone(), w["k"].reshape(T, H * D).clone()
+    F.rotary_emb_v2(q, k, cos, sin, D)
+    q1 = F.rotary_emb(w["q"], w["cos"], w["sin"], False, False)
+    k1 = F.rotary_emb(w["k"], w["cos"], w["sin"], False, False)
+    assert_bit_equal(q.reshape(T, H, D).cpu(), q1.cpu(), "query: one fused launch equals the separate operator")
+    assert_bit_equal(k.reshape(T, H, D).cpu(), k1.cpu(), "key: one fused launch equals the separate operator")
+
+
+def test_rotary_v2_argument_errors():
+    q = torch.randn(4, 64, device=DEV)
+    k = torch.randn(4, 32, device=DEV)
+    c = torch.randn(4, 1, 32, device=DEV)
+    with pytest.raises(rt.DiopiException):
+        F.rotary_emb_v2(q, k, c, c, 31)  # odd dim
+    with pytest.raises(rt.DiopiException):
+        F.rotary_emb_v2(q, k, c[:3], c, 32)  # table with the wrong number of tokens
+    with pytest.raises(rt.DiopiException):
+        F.rotary_emb_v2(q, k.half(), c, c, 32)  # mixed dtypes
+
+
 # ----------------------------------------------------------------------------- decode attention
 def _decode_case(w, dtype, what, seq_subset=None):
     """token_attention then token_softmax_reducev on workload dict `w`; oracle on the CPU for `seq_subset` sequences."""

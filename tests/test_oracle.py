@@ -153,6 +153,42 @@ def test_rotary_reference_shapes_broadcast(golden):
             assert abs(float(out[idx + (0,)]) - want) < 1e-5
 
 
+def test_rotary_v2_identity_tables_and_agreement_with_rotary_emb():
+    g = rng(8)
+    T, Hq, Hk, dim = 7, 3, 2, 16
+    for dtype in (torch.float16, torch.bfloat16, torch.float32, torch.float64):
+        q = torch.randn(T, Hq * dim, generator=g).to(dtype)
+        k = torch.randn(T, Hk * dim, generator=g).to(dtype)
+        q2, k2 = O.rotary_emb_v2(q, k, torch.ones(T, 1, dim, dtype=dtype), torch.zeros(T, 1, dim, dtype=dtype), dim)
+        assert_bit_equal(q2, q, "cos = 1, sin = 0 leaves query alone")
+        assert_bit_equal(k2, k, "cos = 1, sin = 0 leaves key alone")
+    # tables with duplicated halves: the operator is rotary_emb (conj = False) on the [T, heads, dim] view
+    q = torch.randn(T, Hq * dim, generator=g, dtype=torch.float64)
+    k = torch.randn(T, Hk * dim, generator=g, dtype=torch.float64)
+    ang = torch.rand(T, 1, dim // 2, generator=g, dtype=torch.float64) * 6.28
+    cos, sin = torch.cat((ang.cos(), ang.cos()), -1), torch.cat((ang.sin(), ang.sin()), -1)
+    q2, k2 = O.rotary_emb_v2(q, k, cos, sin, dim, exact=True)
+    assert_close(q2.reshape(T, Hq, dim), O.rotary_emb(q.reshape(T, Hq, dim), ang.cos(), ang.sin(), False, exact=True), 1e-13, 1e-14, "query vs rotary_emb")
+    assert_close(k2.reshape(T, Hk, dim), O.rotary_emb(k.reshape(T, Hk, dim), ang.cos(), ang.sin(), False, exact=True), 1e-13, 1e-14, "key vs rotary_emb")
+
+
+def test_rotary_v2_python_loops_with_unequal_table_halves():
+    g = rng(9)
+    T, H, dim = 4, 2, 8
+    q = torch.randn(T, H * dim, generator=g, dtype=torch.float64)
+    k = torch.randn(T, dim, generator=g, dtype=torch.float64)
+    cos = torch.randn(T, 1, dim, generator=g, dtype=torch.float64)  # not a rotation: the two halves are unrelated numbers
+    sin = torch.randn(T, 1, dim, generator=g, dtype=torch.float64)
+    q2, k2 = O.rotary_emb_v2(q, k, cos, sin, dim, exact=True)
+    for x, y, heads in ((q, q2, H), (k, k2, 1)):
+        for t in range(T):
+            for h in range(heads):
+                for d in range(dim):
+                    partner = x[t, h * dim + d + dim // 2] * -1.0 if d < dim // 2 else x[t, h * dim + d - dim // 2]
+                    want = x[t, h * dim + d] * cos[t, 0, d] + partner * sin[t, 0, d]
+                    assert abs(float(y[t, h * dim + d]) - float(want)) < 1e-13, (t, h, d)
+
+
 def test_rotary_fp64_is_computed_in_fp32():
     # rotary.cu:30-43 narrows every operand with static_cast<float>, also for double tensors
     x = torch.tensor([1.0 + 2 ** -40, 3.0], dtype=torch.float64)
