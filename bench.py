@@ -44,7 +44,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,cfg3,cfg4,cfg5")
+    ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,penalty,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
@@ -215,6 +215,29 @@ def main():
         record("diopiRotaryEmbeddingV2 (q,k in place, one launch)", "cfg2 bf16 [16384,32,128] x2", ms_r2, 2 * 2 * T * H * D * 2 + 2 * T * D * 2, "hbm", "bf16",
                None, note="widening beyond the seven hot-path operators; bytes = read+write of q and k, full-width cos/sin once")
         del sets, hs
+        torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ sampling penalties on the step's logits
+    if not only or "penalty" in only:
+        import numpy as np
+        Bp, Vp, Lp = 64, 32000, 1024  # 64 sequences, LLaMA vocabulary, 1024 distinct generated ids each
+        rng = np.random.Generator(np.random.PCG64(17))
+        ids = torch.from_numpy(np.concatenate([rng.permutation(Vp)[:Lp] for _ in range(Bp)]).astype(np.int32)).to(dev)
+        cnt = torch.from_numpy(rng.integers(1, 20, size=Bp * Lp).astype(np.int32)).to(dev)
+        cum = torch.arange(0, (Bp + 1) * Lp, Lp, dtype=torch.int32, device=dev)
+        lg = torch.randn(Bp, Vp, device=dev).half()
+        pres, freq = torch.rand(Bp, device=dev).half(), torch.rand(Bp, device=dev).half()
+        hp = {k: Tensor(v) for k, v in dict(lg=lg, pres=pres, freq=freq, ids=ids, cnt=cnt, cum=cum).items()}
+
+        def pen(i):
+            check(impl.diopiApplyPenalty(ctx.handle, hp["lg"].handle, hp["pres"].handle, hp["freq"].handle, hp["ids"].handle, hp["cnt"].handle,
+                                         hp["cum"].handle, Lp), "diopiApplyPenalty")
+
+        ms_p = timed(pen)
+        record("diopiApplyPenalty", "fp16 logits [64,32000], 1024 ids per sequence", ms_p, Bp * Lp * (4 + 4 + 2 + 2), "hbm", "f16", None,
+               note="widening beyond the seven hot-path operators; a 65536-element scatter, bound by launch and memory latency, not bandwidth; "
+                    "bytes = id + count + logit read + logit write per listed token")
+        del hp, lg, ids, cnt
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ decode configurations

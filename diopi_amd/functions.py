@@ -76,6 +76,28 @@ def rotary_emb_v2(query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin
     return query, key
 
 
+def apply_penalty(logits: torch.Tensor, presence_penalty: torch.Tensor, frequency_penalty: torch.Tensor, p_token_ids: torch.Tensor,
+                  p_token_counts: torch.Tensor, p_cumsum_seq_len: torch.Tensor, p_max_len_in_batch: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """In place on logits, like the reference wrapper (diopi_functions.py:7851-7895)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, logits):
+        keep, h = _handles(logits, presence_penalty, frequency_penalty, p_token_ids, p_token_counts, p_cumsum_seq_len)
+        ret = rt.libs().impl.diopiApplyPenalty(ctx.handle, *h, int(p_max_len_in_batch))
+    check_returncode(ret, "diopiApplyPenalty")
+    return logits
+
+
+def apply_penalty_v2(logits: torch.Tensor, presence_penalty: torch.Tensor, frequency_penalty: torch.Tensor, repetition_penalty: torch.Tensor,
+                     p_token_ids: torch.Tensor, p_token_counts: torch.Tensor, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """In place on logits, like the reference wrapper (diopi_functions.py:8019-8049)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, logits):
+        keep, h = _handles(logits, presence_penalty, frequency_penalty, repetition_penalty, p_token_ids, p_token_counts)
+        ret = rt.libs().impl.diopiApplyPenaltyV2(ctx.handle, *h)
+    check_returncode(ret, "diopiApplyPenaltyV2")
+    return logits
+
+
 def rms_norm(input: torch.Tensor, normalized_shape: Sequence[int], weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
              ctx: Optional[rt.Context] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     ctx = _ctx(ctx)

@@ -136,6 +136,8 @@ class _Libs:
         b = ctypes.c_bool
         impl.diopiRotaryEmbedding.argtypes = [vp, vp, vp, vp, vp, b, b]
         impl.diopiRotaryEmbeddingV2.argtypes = [vp, vp, vp, vp, vp, i64]
+        impl.diopiApplyPenalty.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
+        impl.diopiApplyPenaltyV2.argtypes = [vp, vp, vp, vp, vp, vp, vp]
         impl.diopiRMSNorm.argtypes = [vp, vp, vp, vp, _SizeStruct, vp, vp, ctypes.c_double]
         impl.diopiRMSNormBackward.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, _SizeStruct, ctypes.c_double]
         impl.diopiDestIndexCopyKV.argtypes = [vp, vp, vp, vp]
@@ -150,6 +152,8 @@ class _Libs:
 OPERATOR_SYMBOLS = (
     "diopiRotaryEmbedding",
     "diopiRotaryEmbeddingV2",
+    "diopiApplyPenalty",
+    "diopiApplyPenaltyV2",
     "diopiRMSNorm",
     "diopiRMSNormBackward",
     "diopiDestIndexCopyKV",

@@ -51,6 +51,28 @@ DIOPI_API diopiError_t diopiRotaryEmbeddingV2(diopiContextHandle_t ctx, diopiTen
                                               diopiConstTensorHandle_t sin, int64_t dim);
 
 /*
+ * Presence / frequency penalty on the logits of already generated tokens, in place.
+ * reference: functions_ext.h:527-529 (impl/torch/functions/functions_lightllm.cpp:28-51).
+ *   sequence i owns entries [cum[i], cum[i+1]) of p_token_ids / p_token_counts:
+ *   logits[i, id_j] <- logits[i, id_j] - count_j * frequency_penalty[i] - presence_penalty[i]
+ * evaluated left to right in the logits dtype.  logits [batch, vocabulary]; penalties [batch] in the logits dtype;
+ * ids, counts, cumulative lengths int32 or int64.  p_max_len_in_batch is not read (the reference ignores it too).
+ */
+DIOPI_API diopiError_t diopiApplyPenalty(diopiContextHandle_t ctx, diopiTensorHandle_t logits, diopiConstTensorHandle_t presence_penalty,
+                                         diopiConstTensorHandle_t frequency_penalty, diopiConstTensorHandle_t p_token_ids,
+                                         diopiConstTensorHandle_t p_token_counts, diopiConstTensorHandle_t p_cumsum_seq_len, int p_max_len_in_batch);
+
+/*
+ * Repetition / frequency / presence penalty with one penalty entry per generated token, in place.
+ * reference: functions_ext.h:547-549 (statement: customized_test.py:823-841).
+ *   x = logits.view(-1)[id_j];  x <- x > 0 ? x / repetition_j : x * repetition_j;  x <- x - count_j * frequency_j - presence_j
+ * p_token_ids are flat indices into logits; all penalty tensors and p_token_counts have the length of p_token_ids.
+ */
+DIOPI_API diopiError_t diopiApplyPenaltyV2(diopiContextHandle_t ctx, diopiTensorHandle_t logits, diopiConstTensorHandle_t presence_penalty,
+                                           diopiConstTensorHandle_t frequency_penalty, diopiConstTensorHandle_t repetition_penalty,
+                                           diopiConstTensorHandle_t p_token_ids, diopiConstTensorHandle_t p_token_counts);
+
+/*
  * RMS normalisation over the trailing `normalized_shape` dimensions.
  * reference: functions_ext.h:45-46.
  *   inv_rms[row] = rsqrt(mean(x[row]^2) + eps)         (fp32 accumulate; fp64 for fp64 input)

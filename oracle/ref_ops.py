@@ -1,5 +1,5 @@
-"""CPU oracle for the LLaMA-inference operators (the seven of the hot path and
-diopiRotaryEmbeddingV2).  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the LLaMA-inference operators (the seven of the hot path,
+diopiRotaryEmbeddingV2 and diopiApplyPenalty/V2).  TEST INFRASTRUCTURE ONLY.
 
 This module restates, on the CPU with plain ATen (torch) and numpy calls, what the reference
 computes for each operator.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
@@ -16,6 +16,8 @@ rotary_emb                   functions_ext.cpp:43-64, functions_ext/rotary.cu:26
                              customized_test.py:374-390
 rotary_emb_v2                customized_test.py:843-852 (the torch implementation has no body for
                              diopiRotaryEmbeddingV2; declaration functions_ext.h:649-650)
+apply_penalty                functions_lightllm.cpp:28-51; customized_test.py:667-692
+apply_penalty_v2             customized_test.py:823-841 (no torch body; declaration functions_ext.h:547-549)
 destindex_copy_kv            functions_lightllm.cpp:18-26; customized_test.py:694-696
 token_attention              functions_lightllm.cpp:53-80; customized_test.py:698-713
 token_softmax_reducev        functions_lightllm.cpp:82-107; customized_test.py:715-733
@@ -46,6 +48,9 @@ How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"
                        reproduce rotary_emb on the [T, heads, dim] view, explicit Python loops in
                        float64 with tables whose halves differ, the reference's case shape
                        (diopi_configs.py:9107-9135)
+  apply_penalty / v2   the reference's value fixtures (diopi_configs.py:9265-9312, 9468-9515) against results
+                       worked out by hand in exact decimal arithmetic, untouched entries compared bit for
+                       bit, explicit Python loops
   destindex_copy_kv    the reference fixtures dest_loc=(0..4),(14..17) into 120 rows
                        (diopi_configs.py:9321-9333), untouched rows compared byte for byte
   token_attention      the reference's integer fixture (diopi_configs.py:9541-9558) read against an
@@ -153,6 +158,36 @@ def rotary_emb_v2(query: torch.Tensor, key: torch.Tensor, cos: torch.Tensor, sin
         rotated = torch.cat((-x2, x1), dim=-1)
         return (xv * c + rotated * s).reshape(x.shape)
     return one(query), one(key)
+
+
+def apply_penalty(logits: torch.Tensor, presence_penalty: torch.Tensor, frequency_penalty: torch.Tensor, p_token_ids: torch.Tensor,
+                  p_token_counts: torch.Tensor, p_cumsum_seq_len: torch.Tensor, p_max_len_in_batch: int = 0, exact: bool = False) -> torch.Tensor:
+    """functions_lightllm.cpp:39-48, in place on logits (a float64 copy is returned when exact): per sequence i,
+    logits[i, ids] = logits[i, ids] - counts * frequency[i] - presence[i], every step in the logits dtype."""
+    work = logits.to(torch.float64) if exact else logits
+    pres = presence_penalty.to(work.dtype)
+    freq = frequency_penalty.to(work.dtype)
+    for i in range(work.shape[0]):
+        b, e = int(p_cumsum_seq_len[i]), int(p_cumsum_seq_len[i + 1])
+        ids = p_token_ids[b:e].long()
+        cur = work[i].index_select(0, ids)
+        cur = cur - p_token_counts[b:e] * freq[i] - pres[i]
+        work[i, ids] = cur
+    return work
+
+
+def apply_penalty_v2(logits: torch.Tensor, presence_penalty: torch.Tensor, frequency_penalty: torch.Tensor, repetition_penalty: torch.Tensor,
+                     p_token_ids: torch.Tensor, p_token_counts: torch.Tensor, exact: bool = False) -> torch.Tensor:
+    """customized_test.py:823-841, in place on logits (a float64 copy is returned when exact)."""
+    work = logits.to(torch.float64) if exact else logits
+    flat = work.view(-1)
+    ids = p_token_ids.long()
+    pres, freq, rep = (t.to(work.dtype) for t in (presence_penalty, frequency_penalty, repetition_penalty))
+    cur = flat.index_select(0, ids)
+    cur = torch.where(cur > 0, cur / rep, cur * rep)
+    cur = cur - p_token_counts * freq - pres
+    flat[ids] = cur
+    return work
 
 
 def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

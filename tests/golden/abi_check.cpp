@@ -19,6 +19,10 @@ const char* diopiGetLastErrorString();
 diopiError_t diopiRotaryEmbedding(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
                                   const bool, const bool);
 diopiError_t diopiRotaryEmbeddingV2(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, int64_t);
+diopiError_t diopiApplyPenalty(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
+                               diopiConstTensorHandle_t, diopiConstTensorHandle_t, int);
+diopiError_t diopiApplyPenaltyV2(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
+                                 diopiConstTensorHandle_t, diopiConstTensorHandle_t);
 diopiError_t diopiRMSNorm(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiSize_t, diopiConstTensorHandle_t,
                           diopiConstTensorHandle_t, double);
 diopiError_t diopiRMSNormBackward(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t,

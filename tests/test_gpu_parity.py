@@ -316,6 +316,79 @@ def test_rotary_v2_argument_errors():
         F.rotary_emb_v2(q, k.half(), c, c, 32)  # mixed dtypes
 
 
+# ----------------------------------------------------------------------------- sampling penalties
+PENALTY_LOGITS = [[0.1, 0.5, 0.4, 0.3, 0.5], [0.2, 0.4, 0.0, 0.0, 0.0], [0.3, 0.4, 0.5, 0.3, 0.0]]
+PENALTY_COUNTS = [3, 3, 2, 2, 1, 3, 3, 3, 3, 2, 2]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_apply_penalty_reference_fixture_and_random(dtype):
+    dt = TORCH_DTYPES[dtype]
+    for idt in (torch.int32, torch.int64):
+        logits = torch.tensor(PENALTY_LOGITS, dtype=dt, device=DEV)  # diopi_configs.py:9265-9312
+        pres, freq = torch.tensor([0.1, 0.8, 1.0], dtype=dt, device=DEV), torch.tensor([0.3, 0.5, 0.4], dtype=dt, device=DEV)
+        ids = torch.tensor([0, 1, 2, 3, 4, 0, 1, 0, 1, 2, 3], dtype=idt, device=DEV)
+        cnt = torch.tensor(PENALTY_COUNTS, dtype=idt, device=DEV)
+        cum = torch.tensor([0, 5, 7, 11], dtype=idt, device=DEV)
+        want = O.apply_penalty(logits.cpu().clone(), pres.cpu(), freq.cpu(), ids.cpu(), cnt.cpu(), cum.cpu(), 5)
+        before = snapshot(pres, freq, ids, cnt, cum)
+        F.apply_penalty(logits, pres, freq, ids, cnt, cum, 5)
+        assert_unmodified(before, pres, freq, ids, cnt, cum)
+        assert_bit_equal(logits.cpu(), want, f"apply_penalty fixture {dtype} {idt}: the reference's rounding sequence is reproduced exactly")
+    # a batch of 37 sequences over a 32000-entry vocabulary, distinct ids per sequence, one empty sequence
+    rng = np.random.Generator(np.random.PCG64(91))
+    B, V = 37, 32000
+    lens = rng.integers(0, 400, size=B)
+    lens[11] = 0
+    cum = np.concatenate(([0], np.cumsum(lens)))
+    ids = np.concatenate([rng.permutation(V)[:n] for n in lens]).astype(np.int32)
+    cnt = rng.integers(1, 50, size=int(cum[-1])).astype(np.int32)
+    g = gen(92)
+    logits = torch.randn(B, V, generator=g).to(dt).to(DEV)
+    pres, freq = torch.rand(B, generator=g).to(dt).to(DEV), torch.rand(B, generator=g).to(dt).to(DEV)
+    want = O.apply_penalty(logits.cpu().clone(), pres.cpu(), freq.cpu(), torch.from_numpy(ids), torch.from_numpy(cnt), torch.from_numpy(cum.astype(np.int32)), 400)
+    F.apply_penalty(logits, pres, freq, torch.from_numpy(ids).to(DEV), torch.from_numpy(cnt).to(DEV), torch.from_numpy(cum.astype(np.int32)).to(DEV), 400)
+    assert_bit_equal(logits.cpu(), want, f"apply_penalty random batch {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
+def test_apply_penalty_v2_reference_fixture_and_random(dtype):
+    dt = TORCH_DTYPES[dtype]
+    pen = torch.tensor([0.1] * 4 + [0.8] * 4 + [1.0] * 3, dtype=dt, device=DEV)  # diopi_configs.py:9468-9515
+    ids = torch.tensor([0, 1, 2, 3, 4, 5, 6, 8, 9, 10, 11], dtype=torch.int32, device=DEV)
+    cnt = torch.tensor(PENALTY_COUNTS, dtype=torch.int32, device=DEV)
+    logits = torch.tensor(PENALTY_LOGITS, dtype=dt, device=DEV)
+    want = O.apply_penalty_v2(logits.cpu().clone(), pen.cpu(), pen.cpu(), pen.cpu(), ids.cpu(), cnt.cpu())
+    F.apply_penalty_v2(logits, pen, pen, pen, ids, cnt)
+    assert_bit_equal(logits.cpu(), want, f"apply_penalty_v2 fixture {dtype}")
+    rng = np.random.Generator(np.random.PCG64(93))
+    B, V, n = 16, 32000, 5000
+    flat_ids = rng.permutation(B * V)[:n].astype(np.int64)
+    g = gen(94)
+    logits = torch.randn(B, V, generator=g).to(dt).to(DEV)
+    pres, freq = torch.rand(n, generator=g).to(dt).to(DEV), torch.rand(n, generator=g).to(dt).to(DEV)
+    rep = (torch.rand(n, generator=g) + 0.5).to(dt).to(DEV)
+    cnt = torch.from_numpy(rng.integers(1, 50, size=n).astype(np.int32))
+    want = O.apply_penalty_v2(logits.cpu().clone(), pres.cpu(), freq.cpu(), rep.cpu(), torch.from_numpy(flat_ids), cnt)
+    F.apply_penalty_v2(logits, pres, freq, rep, torch.from_numpy(flat_ids).to(DEV), cnt.to(DEV))
+    assert_bit_equal(logits.cpu(), want, f"apply_penalty_v2 random {dtype}")
+
+
+def test_apply_penalty_argument_errors_and_out_of_range_ids():
+    logits = torch.zeros(2, 8, device=DEV)
+    p = torch.ones(2, device=DEV)
+    ids = torch.tensor([1, 100, -3], dtype=torch.int32, device=DEV)  # two ids outside the vocabulary are skipped
+    cnt = torch.ones(3, dtype=torch.int32, device=DEV)
+    F.apply_penalty(logits, p, p, ids, cnt, torch.tensor([0, 2, 3], dtype=torch.int32, device=DEV), 3)
+    want = torch.zeros(2, 8)
+    want[0, 1] = -2.0
+    assert_bit_equal(logits.cpu(), want, "ids outside the vocabulary")
+    with pytest.raises(rt.DiopiException):
+        F.apply_penalty(logits, p, p, ids, cnt, torch.tensor([0, 3], dtype=torch.int32, device=DEV), 3)  # cumulative lengths too short
+    with pytest.raises(rt.DiopiException):
+        F.apply_penalty(logits, p.half(), p, ids, cnt, torch.tensor([0, 2, 3], dtype=torch.int32, device=DEV), 3)  # penalty dtype
+
+
 # ----------------------------------------------------------------------------- decode attention
 def _decode_case(w, dtype, what, seq_subset=None):
     """token_attention then token_softmax_reducev on workload dict `w`; oracle on the CPU for `seq_subset` sequences."""

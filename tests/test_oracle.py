@@ -189,6 +189,56 @@ def test_rotary_v2_python_loops_with_unequal_table_halves():
                     assert abs(float(y[t, h * dim + d]) - float(want)) < 1e-13, (t, h, d)
 
 
+# the reference's value fixtures for the penalty operators (diopi_configs.py:9265-9312 and 9468-9515)
+PENALTY_LOGITS = [[0.1, 0.5, 0.4, 0.3, 0.5], [0.2, 0.4, 0.0, 0.0, 0.0], [0.3, 0.4, 0.5, 0.3, 0.0]]
+PENALTY_COUNTS = [3, 3, 2, 2, 1, 3, 3, 3, 3, 2, 2]
+
+
+def test_apply_penalty_reference_fixture_worked_by_hand():
+    from fractions import Fraction as Fr
+    logits = torch.tensor(PENALTY_LOGITS, dtype=torch.float64)
+    pres, freq = [Fr(1, 10), Fr(8, 10), Fr(1)], [Fr(3, 10), Fr(5, 10), Fr(4, 10)]
+    ids = [0, 1, 2, 3, 4, 0, 1, 0, 1, 2, 3]
+    cum = [0, 5, 7, 11]
+    # exact decimal arithmetic, entry by entry, independent of the oracle's tensor expressions
+    want = [[Fr(str(v)) for v in row] for row in PENALTY_LOGITS]
+    for i in range(3):
+        for j in range(cum[i], cum[i + 1]):
+            want[i][ids[j]] = want[i][ids[j]] - PENALTY_COUNTS[j] * freq[i] - pres[i]
+    assert want[0][0] == Fr(-9, 10) and want[1][1] == Fr(-19, 10) and want[2][3] == Fr(-15, 10) and want[1][2] == 0 and want[2][4] == 0
+    got = O.apply_penalty(logits.clone(), torch.tensor([0.1, 0.8, 1.0], dtype=torch.float64), torch.tensor([0.3, 0.5, 0.4], dtype=torch.float64),
+                          torch.tensor(ids, dtype=torch.int32), torch.tensor(PENALTY_COUNTS, dtype=torch.int32), torch.tensor(cum, dtype=torch.int32), 5)
+    assert_close(got, torch.tensor([[float(v) for v in row] for row in want], dtype=torch.float64), 1e-14, 1e-15, "fixture")
+    # entries no sequence lists keep their bits, also in fp16
+    l16 = torch.tensor(PENALTY_LOGITS, dtype=torch.float16)
+    g16 = O.apply_penalty(l16.clone(), torch.tensor([0.1, 0.8, 1.0]).half(), torch.tensor([0.3, 0.5, 0.4]).half(), torch.tensor(ids, dtype=torch.int32),
+                          torch.tensor(PENALTY_COUNTS, dtype=torch.int32), torch.tensor(cum, dtype=torch.int32), 5)
+    assert_bit_equal(g16[1, 2:], l16[1, 2:], "untouched entries of sequence 1")
+    assert_bit_equal(g16[2, 4:], l16[2, 4:], "untouched entry of sequence 2")
+    assert_close(g16.double(), got, 2e-3, 2e-3, "fp16 follows the float64 result")
+
+
+def test_apply_penalty_v2_reference_fixture_worked_by_hand():
+    from fractions import Fraction as Fr
+    pen = [Fr(1, 10)] * 4 + [Fr(8, 10)] * 4 + [Fr(1)] * 3
+    ids = [0, 1, 2, 3, 4, 5, 6, 8, 9, 10, 11]
+    flat = [Fr(str(v)) for row in PENALTY_LOGITS for v in row]
+    want = list(flat)
+    for j, idx in enumerate(ids):
+        x = flat[idx]
+        x = x / pen[j] if x > 0 else x * pen[j]
+        want[idx] = x - PENALTY_COUNTS[j] * pen[j] - pen[j]
+    assert want[0] == Fr(1) - Fr(3, 10) - Fr(1, 10) and want[7] == flat[7] and want[12] == flat[12]  # 7 and 12..14 are not listed
+    p = torch.tensor([float(v) for v in pen], dtype=torch.float64)
+    got = O.apply_penalty_v2(torch.tensor(PENALTY_LOGITS, dtype=torch.float64), p, p, p, torch.tensor(ids, dtype=torch.int32),
+                             torch.tensor(PENALTY_COUNTS, dtype=torch.int32))
+    assert_close(got.view(-1), torch.tensor([float(v) for v in want], dtype=torch.float64), 1e-13, 1e-15, "fixture v2")
+    # a negative logit is multiplied, not divided
+    neg = O.apply_penalty_v2(torch.tensor([[-2.0, 3.0]], dtype=torch.float64), torch.zeros(2, dtype=torch.float64), torch.zeros(2, dtype=torch.float64),
+                             torch.tensor([4.0, 4.0], dtype=torch.float64), torch.tensor([0, 1]), torch.tensor([0, 0]))
+    assert_close(neg, torch.tensor([[-8.0, 0.75]], dtype=torch.float64), 0, 0, "sign rule")
+
+
 def test_rotary_fp64_is_computed_in_fp32():
     # rotary.cu:30-43 narrows every operand with static_cast<float>, also for double tensors
     x = torch.tensor([1.0 + 2 ** -40, 3.0], dtype=torch.float64)
