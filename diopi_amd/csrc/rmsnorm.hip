@@ -259,129 +259,168 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 
 // ---------------------------------------------------------------------------
 // Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
-// A work-group is GROUPS row teams of 256 threads; team g takes rows row0+g, row0+g+GROUPS, ...
-// Thread t of a team owns packets t, t+256, ... of every row its team visits.  The column sums for
-// grad_weight / grad_bias live in LDS, one private array per team (ds_add, no return value needed), which
-// keeps them out of the register file: the registers hold the current row and the prefetched next row
-// instead, so loads stay in flight across the one barrier per row step (the row sum s[r] crosses the
-// team's four waves through LDS).  At the end the team arrays are summed in a fixed order into one
-// partial row per work-group.  One large work-group per compute unit keeps the partial buffer at one
-// row per unit while 16 waves keep enough loads in flight.
+// A work-group is GROUPS row teams of 256 threads.  In step i, team g of work-group b takes row
+// (i * gridDim.x + b) * GROUPS + g: at any moment the whole grid works on one contiguous window of
+// gridDim.x * GROUPS rows of each tensor, which spreads the traffic evenly over the memory channels (a private run of
+// rows per work-group would put the work-groups, which advance in step, a fixed large stride apart).
+// Thread t of a team owns packets t, t+256, ... of every row its team visits.
+//
+// Rows travel through buffer loads and stores whose descriptor covers exactly one row (and nothing for a row past
+// the end of the work-group's run): packets beyond the row read as zero and stores to them are dropped by the
+// hardware, so the row loop has no branch around a memory instruction.  A team keeps two rows in registers: while
+// the row of step i is reduced and written back, the row of step i+1 is already there and the row of step i+2 is
+// requested into the registers the first one leaves.  The first step is peeled off the loop so that every later step sees the same sequence of
+// outstanding memory operations (one row of loads, the stores of the previous step, the next row of loads) and only
+// waits for the oldest of them.
+//
+// The column sums for grad_weight / grad_bias are accumulated in fp32 registers and moved every kBwdFlush steps into
+// per-team LDS arrays of ColAcc (fp64 for fp32 tensors), which bounds the length of any fp32 summation; at the end
+// the team arrays are summed in a fixed order into one partial row per work-group.  One large work-group per compute
+// unit keeps the partial buffer at one row per unit.  The row sum s[r] crosses the team's four waves through LDS:
+// one barrier per step.
 // ---------------------------------------------------------------------------
 constexpr int kBwdTeam = 256;
 constexpr int kBwdTeamWaves = kBwdTeam / kWave;
+constexpr int kBwdFlush = 8;
+constexpr int kBufferWord3 = 0x00020000;  // raw buffer, 32-bit data format
+constexpr int kBufferStream = 2;          // cache policy: non-temporal
+
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rowBuffer(const T* base, int64_t row, int n2, bool valid) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base + row * n2), 0, valid ? n2 * static_cast<int>(sizeof(T)) : 0, kBufferWord3);
+}
 
 template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS>
 __global__ __launch_bounds__(kBwdTeam* GROUPS) void rmsNormBwdFused(T* __restrict__ gradInput, ColAcc* __restrict__ partW, ColAcc* __restrict__ partB,
                                                                        const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
-                                                                       const float* __restrict__ invRms, int64_t n1, int n2, int rowsPerBlock) {
+                                                                       const float* __restrict__ invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
     constexpr int kCols = NVT * kBwdTeam * EPV;  // columns covered by the register tiling
     __shared__ float red[2][GROUPS][kBwdTeamWaves];
     extern __shared__ __attribute__((aligned(16))) unsigned char dynLds[];
     // [array(W,B)][team][(j*EPV + e)][tid]: lanes of a wave hit consecutive words
     ColAcc* sAcc = reinterpret_cast<ColAcc*>(dynLds);
-    const int team = threadIdx.x / kBwdTeam;
+    const int team = __builtin_amdgcn_readfirstlane(threadIdx.x / kBwdTeam);  // the same for all lanes of a wave
     const int tid = threadIdx.x % kBwdTeam;
     const int lane = tid % kWave;
     const int wave = tid / kWave;
-    const int nvec = n2 / EPV;
     ColAcc* myW = sAcc + team * kCols;
     ColAcc* myB = sAcc + (GROUPS + team) * kCols;
 
-    float w[NVT][EPV];
+    const int64_t rowsPerStep = static_cast<int64_t>(gridDim.x) * GROUPS;
+    const int steps = static_cast<int>((n1 + rowsPerStep - 1) / rowsPerStep);  // the same for every work-group
+    auto rowOf = [&](int i) { return (static_cast<int64_t>(i) * gridDim.x + blockIdx.x) * GROUPS + team; };
+
+    struct RowRegs {
+        Pack16<T> x[NVT], d[NVT];
+        float inv;
+    };
+    auto request = [&](RowRegs& r, int64_t row) {
+        const bool valid = row < n1;
+        const __amdgpu_buffer_rsrc_t bx = rowBuffer(x, row, n2, valid);
+        const __amdgpu_buffer_rsrc_t bd = rowBuffer(dout, row, n2, valid);
 #pragma unroll
-    for (int j = 0; j < NVT; ++j) {
-        const int v = j * kBwdTeam + tid;
+        for (int j = 0; j < NVT; ++j) {
+            const int off = (j * kBwdTeam + tid) * 16;
+            r.x[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bx, off, 0, kBufferStream);
+            r.d[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bd, off, 0, kBufferStream);
+        }
+        r.inv = invRms[valid ? row : 0];  // uniform address: a scalar load, no branch
+    };
+
+    // the weight packets are requested before the rows: a wait for the first row then covers them as well
+    Pack16<T> wv[NVT];
+    {
+        const __amdgpu_buffer_rsrc_t bw = rowBuffer(weight, 0, n2, true);
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-            w[j][e] = (v < nvec) ? toFloat(weight[v * EPV + e]) : 0.f;
-            myW[(j * EPV + e) * kBwdTeam + tid] = 0;
-            if (HAS_GBIAS) myB[(j * EPV + e) * kBwdTeam + tid] = 0;
+        for (int j = 0; j < NVT; ++j) wv[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bw, (j * kBwdTeam + tid) * 16, 0, 0);
+    }
+    RowRegs ra, rb;
+    request(ra, rowOf(0));
+    request(rb, rowOf(1));
+
+    float w[NVT][EPV], accW[NVT][EPV], accB[HAS_GBIAS ? NVT : 1][EPV];
+    {
+#pragma unroll
+        for (int j = 0; j < NVT; ++j) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                w[j][e] = toFloat(wv[j].e[e]);
+                accW[j][e] = 0.f;
+                if (HAS_GBIAS) accB[j][e] = 0.f;
+                myW[(j * EPV + e) * kBwdTeam + tid] = 0;
+                if (HAS_GBIAS) myB[(j * EPV + e) * kBwdTeam + tid] = 0;
+            }
         }
     }
-
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * rowsPerBlock;
-    int64_t rowEnd = row0 + rowsPerBlock;
-    if (rowEnd > n1) rowEnd = n1;
-    const float fH = static_cast<float>(n2);
-    int parity = 0;
-    // The rows of the next step are requested before the current step is reduced and written back.
-    Pack16<T> xv[NVT], dv[NVT], xn[NVT], dn[NVT];
-    float inv = 0.f, invNext = 0.f;
-    auto request = [&](int64_t row, Pack16<T>* xb, Pack16<T>* db, float* invp) {
-        if (row < rowEnd) {
-            const T* xr = x + row * n2;
-            const T* dr = dout + row * n2;
+    // registers -> this team's LDS arrays; each (team, column) word has exactly one writer
+    auto flush = [&]() {
 #pragma unroll
-            for (int j = 0; j < NVT; ++j) {
-                const int v = j * kBwdTeam + tid;
-                if (v < nvec) {
-                    xb[j] = loadPackStream(xr + v * EPV);
-                    db[j] = loadPackStream(dr + v * EPV);
+        for (int j = 0; j < NVT; ++j) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                myW[(j * EPV + e) * kBwdTeam + tid] += static_cast<ColAcc>(accW[j][e]);
+                accW[j][e] = 0.f;
+                if (HAS_GBIAS) {
+                    myB[(j * EPV + e) * kBwdTeam + tid] += static_cast<ColAcc>(accB[j][e]);
+                    accB[j][e] = 0.f;
                 }
             }
-            *invp = invRms[row];
         }
     };
-    request(row0 + team, xv, dv, &inv);
-    // every team runs the same number of steps so that the barrier below is reached by all of them
-    for (int64_t base = row0; base < rowEnd; base += GROUPS, parity ^= 1) {
-        const int64_t row = base + team;
-        const bool live = row < rowEnd;
-        request(row + GROUPS, xn, dn, &invNext);
+
+    const float fH = static_cast<float>(n2);
+    // One row step of a team on the registers r; rows past the end arrive as zeros and their stores are dropped.
+    auto step = [&](RowRegs& r, int i) {
+        const int64_t row = rowOf(i);
+        const float inv = r.inv;
         float s = 0.f;
-        if (live) {
 #pragma unroll
-            for (int j = 0; j < NVT; ++j) {
-                const int v = j * kBwdTeam + tid;
-                if (v < nvec) {
+        for (int j = 0; j < NVT; ++j) {
 #pragma unroll
-                    for (int e = 0; e < EPV; ++e) {
-                        const float cx = toFloat(xv[j].e[e]);
-                        const float cd = toFloat(dv[j].e[e]);
-                        s += cd * w[j][e] * cx * inv;
-                        // each (team, column) word has exactly one writer: the add is a plain read-modify-write done by the LDS unit
-                        atomicAdd(&myW[(j * EPV + e) * kBwdTeam + tid], static_cast<ColAcc>(cd * cx * inv));
-                        if (HAS_GBIAS) atomicAdd(&myB[(j * EPV + e) * kBwdTeam + tid], static_cast<ColAcc>(cd));
-                    }
-                }
+            for (int e = 0; e < EPV; ++e) {
+                const float cx = toFloat(r.x[j].e[e]);
+                const float cd = toFloat(r.d[j].e[e]);
+                s += cd * w[j][e] * cx * inv;
+                accW[j][e] += cd * cx * inv;
+                if (HAS_GBIAS) accB[j][e] += cd;
             }
         }
         s = waveSum(s);
-        if (lane == 0) red[parity][team][wave] = s;
+        if (lane == 0) red[i & 1][team][wave] = s;
         __syncthreads();
-        if (live) {
-            float sum2 = 0.f;
+        float sum2 = 0.f;
 #pragma unroll
-            for (int i = 0; i < kBwdTeamWaves; ++i) sum2 += red[parity][team][i];
-            const float term1 = (1.0f / fH) * inv;
-            T* gr = gradInput + row * n2;
-#pragma unroll
-            for (int j = 0; j < NVT; ++j) {
-                const int v = j * kBwdTeam + tid;
-                if (v < nvec) {
-                    Pack16<T> gv;
-#pragma unroll
-                    for (int e = 0; e < EPV; ++e) {
-                        const float cx = toFloat(xv[j].e[e]);
-                        const float cd = toFloat(dv[j].e[e]);
-                        float f = fH * cd * w[j][e];
-                        f -= cx * inv * sum2;
-                        f *= term1;
-                        gv.e[e] = fromFloat<T>(f);
-                    }
-                    storePackStream(gr + v * EPV, gv);
-                }
-            }
-        }
+        for (int k = 0; k < kBwdTeamWaves; ++k) sum2 += red[i & 1][team][k];
+        const float term1 = (1.0f / fH) * inv;
+        const __amdgpu_buffer_rsrc_t bg = rowBuffer(gradInput, row, n2, row < n1);
 #pragma unroll
         for (int j = 0; j < NVT; ++j) {
-            xv[j].raw = xn[j].raw;
-            dv[j].raw = dn[j].raw;
+            Pack16<T> gv;
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                const float cx = toFloat(r.x[j].e[e]);
+                const float cd = toFloat(r.d[j].e[e]);
+                float f = fH * cd * w[j][e];
+                f -= cx * inv * sum2;
+                f *= term1;
+                gv.e[e] = fromFloat<T>(f);
+            }
+            __builtin_amdgcn_raw_buffer_store_b128(gv.raw, bg, (j * kBwdTeam + tid) * 16, 0, kBufferStream);
         }
-        inv = invNext;
+        request(r, rowOf(i + 2));
+        if ((i % kBwdFlush) == kBwdFlush - 1) flush();
+    };
+
+    step(ra, 0);  // n1 > 0: there is at least one step
+    // whole pairs in the loop (no exit between the two halves, so both see one fixed sequence of outstanding operations)
+    int i = 1;
+    for (; i + 1 < steps; i += 2) {
+        step(rb, i);
+        step(ra, i + 1);
     }
+    if (i < steps) step(rb, i);
+    flush();
 
     // one partial row per work-group: the team arrays are added in team order
     __syncthreads();
@@ -403,23 +442,26 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS) void rmsNormBwdFused(T* __restric
     }
 }
 
-// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias) in fp64.  A 256-thread group
-// covers 64 columns x 4 slices of the partial rows; lanes of a wave read consecutive columns.
+// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias) in fp64.  A 256-thread group covers
+// kCols = 128 bytes of consecutive columns x (256 / kCols) slices of the partial rows, so that n2 = 4096 spreads over
+// 128 (fp32 partials) or 256 (fp64 partials) work-groups.
 template <typename T, typename ColAcc>
 __global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight, T* __restrict__ gradBias, const ColAcc* __restrict__ partW,
                                                        const ColAcc* __restrict__ partB, int numParts, int n2) {
-    __shared__ double red[2][4][64];
-    const int lane = threadIdx.x % 64;
-    const int slice = threadIdx.x / 64;
-    const int col = blockIdx.x * 64 + lane;
+    constexpr int kCols = 128 / static_cast<int>(sizeof(ColAcc));
+    constexpr int kSlices = 256 / kCols;
+    __shared__ double red[2][kSlices][kCols];
+    const int c = threadIdx.x % kCols;
+    const int slice = threadIdx.x / kCols;
+    const int col = blockIdx.x * kCols + c;
     double sw = 0.0, sb = 0.0;
     if (col < n2) {
         constexpr int kBatch = 8;  // loads of a batch are independent and in flight together
-        for (int p0 = slice; p0 < numParts; p0 += 4 * kBatch) {
+        for (int p0 = slice; p0 < numParts; p0 += kSlices * kBatch) {
             ColAcc vw[kBatch], vb[kBatch];
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                const int p = p0 + 4 * u;
+                const int p = p0 + kSlices * u;
                 vw[u] = p < numParts ? partW[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
                 vb[u] = (gradBias != nullptr && p < numParts) ? partB[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
             }
@@ -430,16 +472,19 @@ __global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight
             }
         }
     }
-    red[0][slice][lane] = sw;
-    red[1][slice][lane] = sb;
+    red[0][slice][c] = sw;
+    red[1][slice][c] = sb;
     __syncthreads();
     if (slice == 0 && col < n2) {
-        sw = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
-        gradWeight[col] = fromDouble<T>(sw);
-        if (gradBias != nullptr) {
-            sb = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
-            gradBias[col] = fromDouble<T>(sb);
+        sw = 0.0;
+        sb = 0.0;
+#pragma unroll
+        for (int k = 0; k < kSlices; ++k) {
+            sw += red[0][k][c];
+            sb += red[1][k][c];
         }
+        gradWeight[col] = fromDouble<T>(sw);
+        if (gradBias != nullptr) gradBias[col] = fromDouble<T>(sb);
     }
 }
 
@@ -620,14 +665,14 @@ diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const Tenso
 // beyond the 64 KiB static limit, which has to be granted per kernel once.
 template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS>
 diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, ColAcc* partW, ColAcc* partB, const T* dout, const T* in, const T* w,
-                               const float* invRms, int64_t n1, int n2, int rowsPerBlock) {
+                               const float* invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
     constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * kBwdTeam * EPV * sizeof(ColAcc);
     auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS>;
     static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                     static_cast<int>(ldsBytes));
     ROCM_HIP(granted);
-    hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2, rowsPerBlock);
+    hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
@@ -646,18 +691,15 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
     const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
     const int groups = gBias ? 2 : 4;
-    // one work-group per compute unit, each walking a contiguous run of rows
+    // one work-group per compute unit (fewer when there are not enough rows to give every team one)
     const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * envInt("DIOPI_ROCM_RMSBWD_BLOCKS_PER_CU", 1);
-    int64_t rowsPerBlock = ceilDiv(d.n1, maxBlocks);
-    rowsPerBlock = ceilDiv(rowsPerBlock, groups) * groups;
-    const int numParts = static_cast<int>(ceilDiv(d.n1, rowsPerBlock));
+    const int numParts = static_cast<int>(std::min<int64_t>(maxBlocks, ceilDiv(d.n1, groups)));
     const int n2 = static_cast<int>(d.n2);
     const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(ColAcc);
     void* scratch = nullptr;
     ROCM_CALL(requireScratch(ctx, partBytes * (gBias ? 2 : 1), &scratch));
     ColAcc* partW = static_cast<ColAcc*>(scratch);
     ColAcc* partB = gBias ? partW + static_cast<int64_t>(numParts) * n2 : nullptr;
-    const int rpb = static_cast<int>(rowsPerBlock);
     T* pgi = static_cast<T*>(gIn.data);
     const T* pdo = static_cast<const T*>(dout.data);
     const T* pin = static_cast<const T*>(in.data);
@@ -666,9 +708,9 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
 #define ROCM_BWD_CASE(NVC)                                                                                                          \
     if constexpr (NVC <= kMaxNvt) {                                                                                                 \
         if (gBias != nullptr) {                                                                                                     \
-            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, true, 2>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2, rpb)));  \
+            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, true, 2>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)));  \
         } else {                                                                                                                    \
-            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, false, 4>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2, rpb))); \
+            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, false, 4>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2))); \
         }                                                                                                                           \
     }
     if (nvt <= 1) {
@@ -679,7 +721,8 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
         ROCM_BWD_CASE(4)
     }
 #undef ROCM_BWD_CASE
-    hipLaunchKernelGGL((rmsNormBwdFold<T, ColAcc>), dim3(static_cast<unsigned>(ceilDiv(n2, 64))), dim3(256), 0, stream, static_cast<T*>(gW.data),
+    constexpr int kFoldCols = 128 / static_cast<int>(sizeof(ColAcc));
+    hipLaunchKernelGGL((rmsNormBwdFold<T, ColAcc>), dim3(static_cast<unsigned>(ceilDiv(n2, kFoldCols))), dim3(256), 0, stream, static_cast<T*>(gW.data),
                        static_cast<T*>(gBias), partW, partB, numParts, n2);
     ROCM_LAUNCH_CHECK();
     *launched = true;
