@@ -131,6 +131,32 @@ __device__ __forceinline__ int64_t loadIndex(const void* base, int64_t i, bool i
     return is64 ? reinterpret_cast<const int64_t*>(base)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(base)[i]);
 }
 
+// The same without a branch: two loads whatever the width (for 32-bit storage the second one re-reads the element),
+// combined afterwards.  A load inside a branch makes the compiler wait for it before the branch ends; this form lets
+// the value stay in flight until its first use.
+__device__ __forceinline__ int64_t loadIndexInFlight(const void* base, int64_t i, bool is64) {
+    const char* p = reinterpret_cast<const char*>(base) + i * (is64 ? 8 : 4);
+    const uint32_t lo = *reinterpret_cast<const uint32_t*>(p);
+    const uint32_t hi = *reinterpret_cast<const uint32_t*>(p + (is64 ? 4 : 0));
+    return is64 ? static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo) : static_cast<int64_t>(static_cast<int32_t>(lo));
+}
+
+// A pointer every lane of the wave holds the same value of, moved to scalar registers (buffer descriptors live there).
+template <typename T>
+__device__ __forceinline__ T* uniformPointer(T* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return reinterpret_cast<T*>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Raw buffer descriptor over `bytes` bytes at `base`: loads past the end return zero and stores past it are dropped by
+// the hardware, so a guarded access needs no branch.
+constexpr int kRawBufferWord3 = 0x00020000;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rawBuffer(const void* base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, kRawBufferWord3);
+}
+
 }  // namespace rocm
 
 #endif  // DIOPI_ROCM_CSRC_DEVICE_HPP_

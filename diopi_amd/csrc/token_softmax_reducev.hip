@@ -61,7 +61,9 @@ struct SplitArgs {
 // so the vector-ALU work per V byte does not grow with G.
 // A wave owns (kv head, token range, sequence), i.e. the G query heads of its kv head, and walks the range in
 // sub-tiles of 128 tokens without ever meeting another wave at a barrier:
-//   * logits of the sub-tile: per query head two coalesced loads (lane = token), prefetched one sub-tile ahead;
+//   * logits of the sub-tile: per query head two coalesced loads (lane = token), prefetched one sub-tile ahead
+//     (tokens past the range alias its last one and become -inf by a select): no load sits inside a branch, so all of
+//     them stay in flight until the next sub-tile's softmax;
 //     running maximum / denominator per head are wave-uniform values (DPP row reduction + four lane reads);
 //     the probabilities go to a wave-private LDS tile [G][128 + 8] in the element type;
 //   * cache slots of the next sub-tile are fetched one sub-tile ahead and parked in wave-private LDS;
@@ -138,9 +140,19 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     float* statW = &sStat[wave][0];
     const T* vHead = v + (hk + (HPW == 1 ? 0 : q)) * kD + c * 8;
     const int64_t colBase = start + t0;
-    const T* xBase = logits + static_cast<int64_t>(hk) * G * a.logitCols + colBase;
+    // tokens of the range whose logits exist: the range may stick out of the logits columns only on invalid input
+    int nLogit = 0;
+    if (colBase >= 0 && colBase < a.logitCols) nLogit = (a.logitCols - colBase < nTokR) ? static_cast<int>(a.logitCols - colBase) : nTokR;
+    // descriptor over the G logits rows of this kv head, from the first column of the range to the last valid one of
+    // row G-1 (the launcher checks that this extent fits 31 bits); empty when no logit of the range exists
+    const int xRowBytes = static_cast<int>(a.logitCols) * static_cast<int>(sizeof(T));
+    const __amdgpu_buffer_rsrc_t xBuf = rawBuffer(uniformPointer(logits + static_cast<int64_t>(hk) * G * a.logitCols + colBase),
+                                                  nLogit > 0 ? (R - 1) * xRowBytes + nLogit * static_cast<int>(sizeof(T)) : 0);
 
-    // logits of sub-tile `sub`: xr[g][k] = logit of query head g, token 64k + lane (-inf outside the sequence)
+    // logits of sub-tile `sub`: xr[g][k] = logit of query head g, token 64k + lane (-inf outside the range).  Lanes
+    // past the range re-read its last token (same cache line, nothing new is fetched) and select -inf; rows g >= R
+    // re-read row 0 and are never looked at.  No condition guards a load: a guarded load is waited for on the spot,
+    // an unguarded one stays in flight until the next sub-tile's softmax.
     float xr[GC][2];
     auto loadLogits = [&](int sub) {
 #pragma unroll
@@ -148,27 +160,39 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
                 const int t = sub * kSub + 64 * k + lane;
-                const int64_t col = colBase + t;
-                xr[g][k] = -INFINITY;
-                if (g < R && t < nTokR && col >= 0 && col < a.logitCols) xr[g][k] = static_cast<float>(xBase[static_cast<int64_t>(g) * a.logitCols + t]);
+                const int tc = t < nLogit ? t : nLogit - 1;
+                const unsigned short raw =
+                    __builtin_amdgcn_raw_buffer_load_b16(xBuf, (g < R ? g : 0) * xRowBytes + tc * static_cast<int>(sizeof(T)), 0, 0);
+                xr[g][k] = (t < nLogit) ? static_cast<float>(__builtin_bit_cast(T, raw)) : -INFINITY;
             }
         }
     };
-    int32_t slotNext[2];
+    // Slot numbers of a sub-tile: requested as raw words through a descriptor over this range of b_loc (element j of a
+    // 64-bit tensor is the word pair at byte 8j; for 32-bit storage the second read repeats the first) and only put
+    // together, clamped and parked in LDS when the rows are about to be requested, so that the reads stay in flight
+    // behind the logits instead of being waited for on the spot.
+    const int locElem = a.loc64 ? 8 : 4;
+    const __amdgpu_buffer_rsrc_t locBuf =
+        rawBuffer(uniformPointer(reinterpret_cast<const char*>(a.bLoc) + locBase * locElem), nTokR * locElem);
+    uint32_t slotLo[2], slotHi[2];
     auto loadSlots = [&](int sub) {
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
             int t = sub * kSub + 64 * k + lane;
             t = t < nTokR ? t : nTokR - 1;  // tokens past the end alias the last valid one (their probability is zero)
-            int64_t slot = loadIndex(a.bLoc, locBase + t, a.loc64);
-            slot = slot < 0 ? 0 : (slot >= a.numSlots ? a.numSlots - 1 : slot);
-            slotNext[k] = static_cast<int32_t>(slot);
+            slotLo[k] = __builtin_amdgcn_raw_buffer_load_b32(locBuf, t * locElem, 0, 0);
+            slotHi[k] = __builtin_amdgcn_raw_buffer_load_b32(locBuf, t * locElem, a.loc64 ? 4 : 0, 0);
         }
     };
     auto storeSlots = [&]() {
         waveLdsFence();
-        slotW[lane] = slotNext[0];
-        slotW[64 + lane] = slotNext[1];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            int64_t slot = a.loc64 ? static_cast<int64_t>((static_cast<uint64_t>(slotHi[k]) << 32) | slotLo[k])
+                                   : static_cast<int64_t>(static_cast<int32_t>(slotLo[k]));
+            slot = slot < 0 ? 0 : (slot >= a.numSlots ? a.numSlots - 1 : slot);
+            slotW[64 * k + lane] = static_cast<int32_t>(slot);
+        }
         waveLdsFence();
     };
     u32x4 rowsV[8];
@@ -181,10 +205,12 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
         for (int r = 0; r < 8; ++r) rowsV[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(sidx[r]) * rowStride));
     };
 
+    // the first logits are requested before the first rows: the softmax of sub-tile 0 then only waits for them, as
+    // the softmax of every later sub-tile does, while rows are in flight
     loadSlots(0);
+    loadLogits(0);
     storeSlots();
     issueV(0);
-    loadLogits(0);
 
     f32x4 acc[8];
 #pragma unroll
@@ -218,10 +244,10 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
                 if (lane == 0) statW[g] = alpha;
             }
         }
-        if (sub + 1 < nSub) {
-            loadLogits(sub + 1);
-            loadSlots(sub + 1);
-        }
+        // requested for every sub-tile, also the last one (nothing past the range is fetched: the reads alias the last
+        // token), so that no load sits inside a branch
+        loadLogits(sub + 1);
+        loadSlots(sub + 1);
         waveLdsFence();
         if (moved) {
             const f32x4 al = *reinterpret_cast<const f32x4*>(statW + 4 * q);
@@ -232,7 +258,9 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
         // A operand: row c, the 8 tokens of this lane group's k slots; rows of other kv heads contribute zeros
         const bool rowLive = HPW == 1 ? c < G : (c < R && c / G == q);
         const T* pRow = tile + (c < R ? c : 0) * kTilePitch + (HPW == 1 ? 8 * q : 0);
-        for (int s = 0; s < nSteps; ++s) {
+        // step 0 runs outside the loop: it waits for rows requested before the softmax and the prefetches above, the
+        // later steps for rows requested one step earlier; in one loop the compiler would make every step wait for all
+        auto pvStep = [&](int s) {
             union {
                 u32x4 u;
                 Frag f;
@@ -261,7 +289,9 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
                 storeSlots();
                 issueV(0);
             }
-        }
+        };
+        pvStep(0);
+        for (int s = 1; s < nSteps; ++s) pvStep(s);
     }
 
     // ---- hand the denominators to the lanes that hold the matching accumulator rows, then store ----
@@ -497,9 +527,10 @@ extern "C" diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t c
 
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    // the matrix-core kernel keeps slot numbers in 32 bits and reads V rows with 16-byte loads
+    // the matrix-core kernel keeps slot numbers in 32 bits, reads V rows with 16-byte loads and addresses the G logits
+    // rows of a kv head with a 32-bit byte offset
     const bool mfma = a.D == kD && a.G <= 16 && a.numSlots < (int64_t(1) << 31) && (reinterpret_cast<uintptr_t>(vV.data) & 15) == 0 &&
-                      envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+                      a.logitCols * 16 * 2 < (int64_t(1) << 31) && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
     switch (vOut.dtype) {
         case diopi_dtype_float16:
             return mfma ? launchWave<half_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)
