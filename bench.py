@@ -34,8 +34,8 @@ WARM_SECONDS = 0.3          # untimed load before every timed region (clock ramp
 # by what it reads for a plain copy of known size (the 65536-row DestIndexCopyKV sweep: 1.9854 KiB per FETCH_SIZE
 # count, 1.0000 KiB per WRITE_SIZE count).  The counters cannot be read from inside this script.
 MEASURED_TRAFFIC_CFG3 = {
-    "tokenAttStaged": int((314577.1 * 1.9854 + 5569.2) * 1024),
-    "softmaxReduceVWave+Merge": int(((315472.4 + 1684.0) * 1.9854 + 2973.8 + 512.0) * 1024),
+    "tokenAttStaged": int((314021.0 * 1.9854 + 4996.9) * 1024),
+    "softmaxReduceVWave+Merge": int(((316226.9 + 1684.0) * 1.9854 + 2974.4 + 512.0) * 1024),
 }
 
 
