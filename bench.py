@@ -18,6 +18,7 @@ Algorithmic bytes / flops are the formulas in diopi_amd/workloads.py.
 import argparse
 import ctypes
 import json
+import math
 import os
 import sys
 import time
@@ -357,7 +358,24 @@ def main():
             cpu = dict(seconds_sample=round(t, 3), TFLOPs=round(f1 / t / 1e12, 4), cores=cores,
                        sample=f"first {L} rows of the shortest sequence; extrapolated by flops to the full configuration: {t * flops / f1:.1f} s")
         record("diopiContextAttentionInference", f"cfg4 fp16 B=8 T={w4['T']}", ms, flops, "mfma", "f16", cpu)
-        del w4
+
+        # the same tokens through the flash-attention interface: cumulative lengths, 32 query heads over 8 key/value
+        # heads, log-sum-exp output (same flop count: every query head still meets every visible key)
+        cu = torch.cat((w4["b_start_loc"], w4["b_start_loc"][-1:] + w4["b_seq_len"][-1:])).to(torch.int32)
+        k8, v8 = w4["k"][:, :8].contiguous(), w4["v"][:, :8].contiguous()
+        lse = torch.zeros(w4["B"], w4["H"], w4["max_input_len"], dtype=torch.float32, device=dev)
+        hf = {k: Tensor(v) for k, v in dict(cu=cu, k8=k8, v8=v8, lse=lse).items()}
+        scale = 1.0 / math.sqrt(w4["D"])
+
+        def fav(i):
+            check(impl.diopiFlashAttentionVarLen(ctx.handle, h["out"].handle, hf["lse"].handle, None, h["q"].handle, hf["k8"].handle, hf["v8"].handle,
+                                                 hf["cu"].handle, hf["cu"].handle, None, w4["max_input_len"], w4["max_input_len"], 0.0, scale, True, -1, -1),
+                  "diopiFlashAttentionVarLen")
+
+        ms_f = timed(fav)
+        record("diopiFlashAttentionVarLen (causal, 32 heads over 8 kv heads, lse)", f"cfg4 tokens fp16 B=8 T={w4['T']}", ms_f, flops, "mfma", "f16", None,
+               note="widening beyond the seven hot-path operators; the prefill kernel in its general form")
+        del w4, hf, k8, v8, lse
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ the JSON line

@@ -25,6 +25,12 @@
 // of the 64 accumulator registers out of the common path.
 // Work-groups are numbered so that the query tiles of one head land on the same XCD (they share that head's K/V
 // through its L2); a small planning kernel orders the tiles of a head longest first.
+//
+// The same kernels serve diopiFlashAttentionVarLen (proto/include/diopi/functions_ext.h:355-359; Python statement
+// customized_test.py:525-588 with multi_head_attention_inside, 36-57): sequences given by cumulative lengths, G query
+// heads per key/value head, an explicit softmax scale, causal or full attention, and the row-wise log-sum-exp as a
+// second output.  That form is a template flag (GEN): the lightllm operator keeps its literal scale and its
+// compile-time causal structure.
 #include <cmath>
 
 #include "common.hpp"
@@ -52,6 +58,13 @@ struct CtxArgs {
     const int2* plan;  // [tilesBound] visiting order of the query tiles of one head, written by ctxAttnPlan
     int tilesBound;    // upper bound on the number of 128-row query tiles over all sequences
     int totalItems;    // H * tilesBound
+    // general form only (diopiFlashAttentionVarLen); the lightllm operator leaves these at their defaults
+    bool cumulative;   // bStartLoc holds batch + 1 cumulative lengths; bSeqLen is unused
+    bool causal;
+    int G;             // query heads per key/value head
+    float scaleLog2;   // softmax scale * log2(e)
+    float* lse;        // [batch, H, lseStride] log-sum-exp of the scaled scores of every query row, or null
+    int lseStride;     // max_seqlen_q
 };
 
 template <typename T>
@@ -83,7 +96,7 @@ struct SeqInfo {
 __device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
     SeqInfo s;
     s.start = loadIndex(a.bStartLoc, i, a.start64);
-    s.len = loadIndex(a.bSeqLen, i, a.len64);
+    s.len = a.cumulative ? loadIndex(a.bStartLoc, i + 1, a.start64) - s.start : loadIndex(a.bSeqLen, i, a.len64);
     if (s.start < 0 || s.start >= a.rows) s.len = 0;
     if (s.len > a.rows - s.start) s.len = a.rows - s.start;
     if (s.len < 0) s.len = 0;
@@ -134,11 +147,13 @@ __global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ p
     }
 }
 
-template <typename T, int NWV>
+template <typename T, int NWV, bool GEN>
 __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                                                                CtxArgs a) {
-    // exp(x / sqrt(D)) = exp2(x * log2(e) / sqrt(D)): one literal factor
-    constexpr float scaleLog2 = 0.12751743082459868f;  // log2(e) / sqrt(128)
+    // exp(x / sqrt(D)) = exp2(x * log2(e) / sqrt(D)): one literal factor (a run-time one in the general form)
+    constexpr float kScaleLog2 = 0.12751743082459868f;  // log2(e) / sqrt(128)
+    const float scaleLog2 = GEN ? a.scaleLog2 : kScaleLog2;
+    const bool causal = GEN ? a.causal : true;
     using Ops = Mfma32<T>;
     using Frag = typename Ops::Frag;
     constexpr int BM = NWV * 32;  // query rows per work-group: each of the NWV waves owns 32 of them
@@ -165,10 +180,12 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     const int wave = tid / kWave;
     const int n = lane % 32;   // query column of this lane in every accumulator
     const int hh = lane / 32;  // which half of the k slots / which 4-row sub-block of the accumulator
-    const int64_t rowPitch = static_cast<int64_t>(a.H) * kHD;
-    const T* qBase = q + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
-    const T* kBase = k + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
-    const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+    const int64_t qPitch = static_cast<int64_t>(a.H) * kHD;                   // row pitch of q and out
+    const int64_t rowPitch = GEN ? static_cast<int64_t>(a.H / a.G) * kHD : qPitch;  // row pitch of k and v
+    const int kvHead = GEN ? head / a.G : head;
+    const T* qBase = q + si.start * qPitch + static_cast<int64_t>(head) * kHD;
+    const T* kBase = k + si.start * rowPitch + static_cast<int64_t>(kvHead) * kHD;
+    const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(kvHead) * kHD;
 
     // ---- Q fragments (B operand of S^T): row = m0 + 32*wave + n, k slot (hh, e) <-> dim 16*s + 8*hh + e ----
     const int qRow = m0 + wave * 32 + n;
@@ -177,7 +194,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
 #pragma unroll
     for (int s = 0; s < kHD / 16; ++s) {
         FragBits<Frag> u;
-        u.raw = *reinterpret_cast<const u32x4*>(qBase + qRowLd * rowPitch + s * 16 + hh * 8);
+        u.raw = *reinterpret_cast<const u32x4*>(qBase + qRowLd * qPitch + s * 16 + hh * 8);
         qf[s] = u.f;
     }
 
@@ -190,7 +207,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     float mRun = -1e30f;
     float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
 
-    const int kEnd = (m0 + BM < L) ? m0 + BM : L;  // keys 0 .. kEnd-1 are visible to this tile
+    const int kEnd = (causal && m0 + BM < L) ? m0 + BM : L;  // keys 0 .. kEnd-1 are visible to this tile
     const int numKeyTiles = (kEnd + kBN - 1) / kBN;
     const int waveRowLo = m0 + wave * 32;
     const int waveRowHi = waveRowLo + 31;
@@ -288,7 +305,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         const T* sVt = sK + kBN * kLD;
 
         const int key0 = jt * kBN;
-        if (key0 > waveRowHi) {
+        if (causal && key0 > waveRowHi) {
             // entirely above the diagonal for this wave: only the staging duty remains
 #pragma unroll
             for (int idx = 0; idx < kPieces; ++idx) stagePiece(idx, jt);
@@ -329,13 +346,16 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         loadV(0, 0);
         __builtin_amdgcn_sched_barrier(0);
         // accumulator register r of block sb holds key  key0 + 32*sb + 8*(r/4) + 4*hh + r%4  for query row qRow
-        if (key0 + kBN - 1 > waveRowLo) {
+        if (causal ? key0 + kBN - 1 > waveRowLo : key0 + kBN > L) {
+            // causal: keys past the query's own position (which covers keys past the sequence, staged as copies of its
+            // last row); full attention: only those
+            const int lastKey = causal ? qRow : L - 1;
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = key0 + sb * 32 + (r / 4) * 8 + hh * 4 + (r % 4);
-                    if (key > qRow) s[sb][r] = -1e30f;
+                    if (key > lastKey) s[sb][r] = -1e30f;
                 }
             }
         }
@@ -398,6 +418,11 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
     const float lTot = lRun + __shfl_xor(lRun, 32, kWave);
     const float inv = 1.0f / lTot;
+    if constexpr (GEN) {
+        // ln sum_j exp(scale * s_j) = ln 2 * (reference maximum in log2 units + log2 of the sum relative to it)
+        if (a.lse != nullptr && hh == 0 && qRow < L && qRow < a.lseStride)
+            a.lse[(static_cast<int64_t>(planned.x) * a.H + head) * a.lseStride + qRow] = 0.6931471805599453f * (mRun * scaleLog2 + __builtin_amdgcn_logf(lTot));
+    }
     __syncthreads();  // the K/V tiles are dead; reuse the storage as a [BM][kLD] output tile
     T* sO = smem;
     static_assert(kHD == 128, "scaleLog2 is written out for head size 128");
@@ -416,7 +441,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     }
     // each wave only reads back the 32 rows it wrote: no work-group barrier needed, LDS ops of a wave are ordered
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    T* oBase = out + si.start * rowPitch + static_cast<int64_t>(head) * kHD;
+    T* oBase = out + si.start * qPitch + static_cast<int64_t>(head) * kHD;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
         const int id = it * kWave + lane;
@@ -425,7 +450,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         const int grow = m0 + wave * 32 + row;
         if (grow < L) {
             const u32x4 val = *reinterpret_cast<const u32x4*>(sO + (wave * 32 + row) * kLD + c * 8);
-            *reinterpret_cast<u32x4*>(oBase + grow * rowPitch + c * 8) = val;
+            *reinterpret_cast<u32x4*>(oBase + grow * qPitch + c * 8) = val;
         }
     }
 }
@@ -447,8 +472,10 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
     if (seq >= a.batch) return;
     const int64_t r = grow - si.start;
     const int lane = threadIdx.x;
-    const int64_t rowPitch = static_cast<int64_t>(a.H) * D;
-    const T* qRow = q + grow * rowPitch + static_cast<int64_t>(head) * D;
+    const int64_t qPitch = static_cast<int64_t>(a.H) * D;
+    const int64_t rowPitch = static_cast<int64_t>(a.H / a.G) * D;  // k and v
+    const int kvHead = head / a.G;
+    const T* qRow = q + grow * qPitch + static_cast<int64_t>(head) * D;
     AccT qv[kPerLane], acc[kPerLane];
 #pragma unroll
     for (int e = 0; e < kPerLane; ++e) {
@@ -457,9 +484,10 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
         acc[e] = 0;
     }
     AccT m = static_cast<AccT>(-INFINITY), l = 0;
-    for (int64_t j = 0; j <= r; ++j) {
-        const T* kRow = k + (si.start + j) * rowPitch + static_cast<int64_t>(head) * D;
-        const T* vRow = v + (si.start + j) * rowPitch + static_cast<int64_t>(head) * D;
+    const int64_t jLast = a.causal ? r : si.len - 1;
+    for (int64_t j = 0; j <= jLast; ++j) {
+        const T* kRow = k + (si.start + j) * rowPitch + static_cast<int64_t>(kvHead) * D;
+        const T* vRow = v + (si.start + j) * rowPitch + static_cast<int64_t>(kvHead) * D;
         AccT part = 0;
 #pragma unroll
         for (int e = 0; e < kPerLane; ++e) {
@@ -478,15 +506,17 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
         }
         m = mNew;
     }
-    T* oRow = out + grow * rowPitch + static_cast<int64_t>(head) * D;
+    T* oRow = out + grow * qPitch + static_cast<int64_t>(head) * D;
 #pragma unroll
     for (int e = 0; e < kPerLane; ++e) {
         const int d = lane + e * kWave;
         if (d < D) oRow[d] = static_cast<T>(acc[e] / l);
     }
+    if (a.lse != nullptr && lane == 0 && r < a.lseStride)
+        a.lse[(static_cast<int64_t>(seq) * a.H + head) * a.lseStride + r] = static_cast<float>(static_cast<double>(m) + log(static_cast<double>(l)));
 }
 
-template <typename T, int NWV>
+template <typename T, int NWV, bool GEN = false>
 diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
     constexpr int BM = NWV * 32;
     a.tilesBound = static_cast<int>(ceilDiv(a.rows, BM)) + a.batch;
@@ -503,24 +533,54 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
     constexpr int ldsBytes = 2 * kStageElems * static_cast<int>(sizeof(T));
-    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
+    static hipError_t granted =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV, GEN>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
     ROCM_HIP(granted);
-    hipLaunchKernelGGL((ctxAttnMfma<T, NWV>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k),
-                       static_cast<const T*>(v), a);
+    hipLaunchKernelGGL((ctxAttnMfma<T, NWV, GEN>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q),
+                       static_cast<const T*>(k), static_cast<const T*>(v), a);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
 
 template <typename T, typename AccT>
-diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const void* v, const CtxArgs& a, int D) {
+diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const void* k, const void* v, const CtxArgs& a, int D, double softmaxScale) {
     ROCM_CHECK(D <= 8 * kWave, "context attention: head size %d is not supported (at most %d)", D, 8 * kWave);
     ROCM_CHECK(a.H <= 65535, "context attention: %d heads exceed the launch limit", a.H);
     ROCM_CHECK(a.rows <= INT32_MAX, "context attention: too many rows for one launch");
-    const AccT scale = static_cast<AccT>(1.0 / std::sqrt(static_cast<double>(D)));
+    const AccT scale = static_cast<AccT>(softmaxScale);
     hipLaunchKernelGGL((ctxAttnGeneric<T, AccT>), dim3(static_cast<unsigned>(a.rows), static_cast<unsigned>(a.H)), dim3(kWave), 0, stream,
                        static_cast<T*>(out), static_cast<const T*>(q), static_cast<const T*>(k), static_cast<const T*>(v), a, D, scale);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
+}
+
+// Picks the kernel for one call: the matrix-core kernel for 16-bit tensors with head size 128 (4 waves per query tile
+// of 128 rows, or 8 waves per 256 rows once the sequences are long enough to fill them), the one-wave-per-row kernel
+// for everything else.  Returns diopiDtypeNotSupported (without a message) for a dtype no kernel takes.
+template <bool GEN>
+diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& vOut, const TensorView& vQ, const TensorView& vK,
+                               const TensorView& vV, const CtxArgs& a, int D, double softmaxScale) {
+    const bool aligned =
+        ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
+    // the planning kernel keeps two ints per sequence and one per query tile in LDS
+    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
+    const bool fast = D == kHD && aligned && planFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    // 256-row query tiles (8 waves share each K/V tile) once the sequences are long enough to fill them
+    const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
+    switch (vQ.dtype) {
+        case diopi_dtype_float16:
+            return fast ? (wide ? launchMfma<half_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                                : launchMfma<half_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
+                        : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
+        case diopi_dtype_bfloat16:
+            return fast ? (wide ? launchMfma<bf16_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
+                                : launchMfma<bf16_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
+                        : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
+        case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
+        case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
+        default: break;
+    }
+    return diopiDtypeNotSupported;
 }
 
 }  // namespace
@@ -564,31 +624,99 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     a.rows = vQ.shape[0];
     a.tilesBound = 0;
     a.totalItems = 0;
+    a.cumulative = false;
+    a.causal = true;
+    a.G = 1;
+    a.scaleLog2 = 0.f;
+    a.lse = nullptr;
+    a.lseStride = 0;
     const int D = static_cast<int>(vQ.shape[2]);
-
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    const bool aligned =
-        ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
-    // the planning kernel keeps two ints per sequence and one per query tile in LDS
-    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
-    const bool fast = D == kHD && aligned && planFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
-    // 256-row query tiles (8 waves share each K/V tile) once the sequences are long enough to fill them
-    const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
-    switch (vQ.dtype) {
-        case diopi_dtype_float16:
-            return fast ? (wide ? launchMfma<half_t, 8>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
-                                : launchMfma<half_t, 4>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
-                        : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
-        case diopi_dtype_bfloat16:
-            return fast ? (wide ? launchMfma<bf16_t, 8>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
-                                : launchMfma<bf16_t, 4>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
-                        : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
-        case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
-        case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D);
-        default: break;
-    }
+    const diopiError_t err = dispatchAttention<false>(ctx, stream, vOut, vQ, vK, vV, a, D, 1.0 / std::sqrt(static_cast<double>(D)));
+    if (err != diopiDtypeNotSupported) return err;
     setLastError("diopiContextAttentionInference: dtype %s is not supported", dtypeName(vQ.dtype));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}
+
+extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                                  diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                                  diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_kv, diopiConstTensorHandle_t alibi_slopes,
+                                                  int32_t max_seqlen_q, int32_t max_seqlen_kv, float p_dropout, float softmax_scale, bool is_causal,
+                                                  int32_t window_size_left, int32_t window_size_right) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;            // only dropout draws random numbers
+    (void)max_seqlen_kv;  // lengths come from the cumulative tensors
+    // the reference's statement covers neither of these (customized_test.py:540 "TODO: impl for alibi and sliding window")
+    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
+        setLastError("diopiFlashAttentionVarLen: dropout, ALiBi slopes and sliding windows are not implemented");
+        return diopiNoImplement;
+    }
+    TensorView vOut, vQ, vK, vV, vCuQ, vCuK, vLse;
+    ROCM_CALL(unwrap(attention_out, "attention_out", &vOut));
+    ROCM_CALL(unwrap(q, "q", &vQ));
+    ROCM_CALL(unwrap(k, "k", &vK));
+    ROCM_CALL(unwrap(v, "v", &vV));
+    ROCM_CALL(unwrap(cum_seq_q, "cum_seq_q", &vCuQ));
+    ROCM_CALL(unwrap(cum_seq_kv, "cum_seq_kv", &vCuK));
+    ROCM_CALL(requireDeviceContiguous(vOut, "attention_out"));
+    ROCM_CALL(requireDeviceContiguous(vQ, "q"));
+    ROCM_CALL(requireDeviceContiguous(vK, "k"));
+    ROCM_CALL(requireDeviceContiguous(vV, "v"));
+    ROCM_CALL(requireDeviceContiguous(vCuQ, "cum_seq_q"));
+    ROCM_CALL(requireDeviceContiguous(vCuK, "cum_seq_kv"));
+    const bool haveLse = softmax_lse != nullptr;
+    if (haveLse) {
+        ROCM_CALL(unwrap(softmax_lse, "softmax_lse", &vLse));
+        ROCM_CALL(requireDeviceContiguous(vLse, "softmax_lse"));
+    }
+    ROCM_CHECK(vQ.ndim == 3 && vK.ndim == 3, "q and k must be [tokens, heads, head_dim], got ranks %d and %d", vQ.ndim, vK.ndim);
+    ROCM_CHECK(vOut.sameShape(vQ) && vV.sameShape(vK), "attention_out must have the shape of q, v the shape of k");
+    // like the reference's statement (customized_test.py:550), queries and keys of a sequence are the same tokens
+    ROCM_CHECK(vK.shape[0] == vQ.shape[0] && vK.shape[2] == vQ.shape[2], "q and k must have the same token count and head size");
+    ROCM_CHECK(vK.shape[1] > 0 && vQ.shape[1] % vK.shape[1] == 0, "the %lld query heads must be a multiple of the %lld key/value heads",
+               static_cast<long long>(vQ.shape[1]), static_cast<long long>(vK.shape[1]));
+    ROCM_CHECK(isFloatDtype(vQ.dtype) && vK.dtype == vQ.dtype && vV.dtype == vQ.dtype && vOut.dtype == vQ.dtype,
+               "q, k, v and attention_out must share one floating dtype (q is %s)", dtypeName(vQ.dtype));
+    ROCM_CHECK(vCuQ.ndim == 1 && vCuQ.shape[0] >= 1 && vCuK.ndim == 1 && vCuK.shape[0] == vCuQ.shape[0] && isIndexDtype(vCuQ.dtype) &&
+                   vCuK.dtype == vCuQ.dtype,
+               "cum_seq_q and cum_seq_kv must be 1-D int32 or int64 tensors of batch + 1 entries");
+    ROCM_CHECK(vCuQ.shape[0] - 1 <= 65535 && vQ.shape[1] <= INT32_MAX / 1024 && vQ.shape[2] <= 65535, "batch / head count / head size out of range");
+    ROCM_CHECK(max_seqlen_q >= 0, "max_seqlen_q must not be negative");
+    const int64_t batch = vCuQ.shape[0] - 1;
+    if (haveLse) {
+        ROCM_CHECK(vLse.dtype == diopi_dtype_float32 && vLse.numel == batch * vQ.shape[1] * static_cast<int64_t>(max_seqlen_q),
+                   "softmax_lse must be float32 [batch, heads, max_seqlen_q] = [%lld, %lld, %d]", static_cast<long long>(batch),
+                   static_cast<long long>(vQ.shape[1]), max_seqlen_q);
+    }
+    if (vQ.numel == 0 || batch == 0) return diopiSuccess;
+
+    CtxArgs a;
+    a.bStartLoc = vCuQ.data;
+    a.bSeqLen = nullptr;
+    a.start64 = vCuQ.dtype == diopi_dtype_int64;
+    a.len64 = a.start64;
+    a.batch = static_cast<int>(batch);
+    a.H = static_cast<int>(vQ.shape[1]);
+    a.rows = vQ.shape[0];
+    a.tilesBound = 0;
+    a.totalItems = 0;
+    a.cumulative = true;
+    a.causal = is_causal;
+    a.G = static_cast<int>(vQ.shape[1] / vK.shape[1]);
+    const int D = static_cast<int>(vQ.shape[2]);
+    // the Python layer passes 1/sqrt(head_dim) for "None" (diopi_functions.py:7564-7566); zero means the same here
+    const double scale = softmax_scale != 0.f ? static_cast<double>(softmax_scale) : 1.0 / std::sqrt(static_cast<double>(D));
+    a.scaleLog2 = static_cast<float>(scale * 1.4426950408889634);
+    a.lse = haveLse ? static_cast<float*>(vLse.data) : nullptr;
+    a.lseStride = max_seqlen_q;
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    const diopiError_t err = dispatchAttention<true>(ctx, stream, vOut, vQ, vK, vV, a, D, scale);
+    if (err != diopiDtypeNotSupported) return err;
+    setLastError("diopiFlashAttentionVarLen: dtype %s is not supported", dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
     ROCM_ENTRY_END
 }

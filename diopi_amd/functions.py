@@ -17,6 +17,8 @@ from __future__ import annotations
 
 from typing import Optional, Sequence
 
+import math
+
 import torch
 
 from . import runtime as rt
@@ -173,4 +175,27 @@ def context_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: to
         keep, h = _handles(out, q, k, v, b_start_loc, b_seq_len)
         ret = rt.libs().impl.diopiContextAttentionInference(ctx.handle, *h, int(max_input_len))
     check_returncode(ret, "diopiContextAttentionInference")
+    return out
+
+
+def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_kv: torch.Tensor, alibi_slopes,
+                           max_seqlen_q: int, max_seqlen_kv: int, p_dropout: float, softmax_scale, is_causal: bool, window_size_left: int = -1,
+                           window_size_right: int = -1, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py:7530-7590 of the reference: allocates out and softmax_lse [batch, heads, max_seqlen_q] (kept in
+    GLOBAL_STATE["flash_attention_varlen_softmax_lse"]), replaces a missing scale by 1/sqrt(head_dim), returns out."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(q)
+    batch = cu_seqlens_q.numel() - 1
+    lse = torch.zeros(batch, q.shape[1], int(max_seqlen_q), dtype=torch.float32, device=q.device)
+    scale = 1.0 / math.sqrt(q.shape[-1]) if not softmax_scale else float(softmax_scale)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, lse, q, k, v, cu_seqlens_q, cu_seqlens_kv)
+        alibi = None
+        if alibi_slopes is not None:
+            keep2, (alibi,) = _handles(alibi_slopes)
+        ret = rt.libs().impl.diopiFlashAttentionVarLen(ctx.handle, h[0], h[1], None, h[2], h[3], h[4], h[5], h[6], alibi, int(max_seqlen_q),
+                                                       int(max_seqlen_kv), float(p_dropout), scale, bool(is_causal), int(window_size_left),
+                                                       int(window_size_right))
+    check_returncode(ret, "diopiFlashAttentionVarLen")
+    GLOBAL_STATE["flash_attention_varlen_softmax_lse"] = lse
     return out

@@ -144,6 +144,8 @@ class _Libs:
         impl.diopiTokenAttentionInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
         impl.diopiTokenSoftmaxReduceVInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32]
         impl.diopiContextAttentionInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
+        impl.diopiFlashAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, ctypes.c_float, ctypes.c_float, ctypes.c_bool,
+                                                   i32, i32]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
@@ -160,6 +162,7 @@ OPERATOR_SYMBOLS = (
     "diopiTokenAttentionInference",
     "diopiTokenSoftmaxReduceVInference",
     "diopiContextAttentionInference",
+    "diopiFlashAttentionVarLen",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

@@ -140,6 +140,23 @@ DIOPI_API diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, 
                                                       diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
                                                       diopiConstTensorHandle_t b_seq_len, int max_input_len);
 
+/*
+ * Variable-length flash attention, forward.
+ * reference: functions_ext.h:355-359 (Python statement customized_test.py:525-588, 36-57).
+ * q [total, Hq, D]; k, v [total, Hkv, D] with Hq a multiple of Hkv (query head h reads key/value head h / (Hq/Hkv));
+ * sequence i owns tokens [cum_seq_q[i], cum_seq_q[i+1]) of q, k and v (cum_seq_kv must describe the same tokens, as in
+ * the reference's statement; it is not read).  attention_out = softmax(softmax_scale * q k^T [+ causal mask]) v,
+ * softmax_lse [batch, Hq, max_seqlen_q] (float32, may be null) receives the log-sum-exp of every query row's scaled
+ * scores; entries past a sequence's length are left untouched.  softmax_scale == 0 means 1/sqrt(D).
+ * Not implemented (error 13): p_dropout != 0, alibi_slopes, sliding windows (window sizes >= 0).  gen is not used.
+ * dtypes: float16, bfloat16 (matrix cores at D == 128), float32, float64; cum_seq int32 or int64.
+ */
+DIOPI_API diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                                 diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                                 diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_kv, diopiConstTensorHandle_t alibi_slopes,
+                                                 int32_t max_seqlen_q, int32_t max_seqlen_kv, float p_dropout, float softmax_scale, bool is_causal,
+                                                 int32_t window_size_left, int32_t window_size_right);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -22,6 +22,8 @@ destindex_copy_kv            functions_lightllm.cpp:18-26; customized_test.py:69
 token_attention              functions_lightllm.cpp:53-80; customized_test.py:698-713
 token_softmax_reducev        functions_lightllm.cpp:82-107; customized_test.py:715-733
 context_attention            functions_lightllm.cpp:109-147; customized_test.py:8-33, 735-749
+flash_attention_varlen       customized_test.py:525-588 with multi_head_attention_inside, 36-57 (the torch
+                             implementation calls the flash-attn library; declaration functions_ext.h:355-359)
 ===========================  =====================================================================
 
 Two arithmetic modes:
@@ -59,6 +61,9 @@ How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"
                        brute force with explicit Python loops
   token_softmax_reducev  constant logits -> mean of the gathered rows, one dominant logit -> that row,
                        L=1 -> the row bit for bit, float64 brute force
+  flash_attention_varlen  causal multi-head case = context_attention on the same tokens, identical keys ->
+                       mean of the visible values and lse = scale*q.k + ln(count), explicit Python loops for
+                       full attention, grouped heads, a custom scale and the log-sum-exp
   context_attention    first token of every sequence returns its v row bit for bit, constant V,
                        the reference's ragged fixtures (diopi_configs.py:9349-9377) incl. untouched
                        rows, float64 brute force, and the last row cross-checked against
@@ -276,3 +281,45 @@ def context_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: to
         end = start + L
         out[start:end] = _torch_context_attention(q[start:end], k[start:end], v[start:end], L, head, dim, exact)
     return out
+
+
+def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_kv: torch.Tensor, alibi_slopes,
+                           max_seqlen_q: int, max_seqlen_kv: int, p_dropout: float, softmax_scale, is_causal: bool, window_size_left: int = -1,
+                           window_size_right: int = -1, exact: bool = False, return_lse: bool = False):
+    """customized_test.py:525-588.  The reference pads every sequence to max_seqlen, adds -10000 to the scores of padded
+    and (if causal) future keys and runs multi_head_attention_inside (36-57): k is scaled in the tensor dtype, scores
+    are an einsum in the tensor dtype, softmax is taken with dtype=v.dtype, the output is an einsum with v.  The shifted
+    keys get weight exp(-10000 + ...) = 0 exactly, so working on each sequence at its own length is the same
+    computation; that is what is done here.  exact=True: float64 throughout with -inf masks, rounded once at the end.
+    return_lse: also returns the float64 log-sum-exp of the scaled visible scores, [batch, heads, max_seqlen_q], zero
+    where a sequence is shorter."""
+    assert alibi_slopes is None and p_dropout == 0 and window_size_left < 0 and window_size_right < 0, "not covered by the reference's statement"
+    hq, hkv, d = q.shape[1], k.shape[1], q.shape[2]
+    g = hq // hkv
+    scale = softmax_scale or 1.0 / math.sqrt(d)
+    batch = cu_seqlens_q.numel() - 1
+    out = torch.zeros_like(q)
+    lse = torch.zeros(batch, hq, int(max_seqlen_q), dtype=torch.float64)
+    for i in range(batch):
+        b, e = int(cu_seqlens_q[i]), int(cu_seqlens_q[i + 1])
+        n = e - b
+        if n == 0:
+            continue
+        qs, ks, vs = q[b:e], k[b:e], v[b:e]
+        if g > 1:  # "... hkv d -> ... (hkv g) d": query head h reads key/value head h // g
+            ks, vs = ks.repeat_interleave(g, dim=1), vs.repeat_interleave(g, dim=1)
+        future = torch.triu(torch.ones(n, n, dtype=torch.bool), 1)
+        q64, k64, v64 = qs.double(), ks.double(), vs.double()
+        s64 = torch.einsum("thd,shd->hts", q64, k64) * scale
+        if is_causal:
+            s64 = s64.masked_fill(future, float("-inf"))
+        lse[i, :, :min(n, int(max_seqlen_q))] = torch.logsumexp(s64, dim=-1)[:, :int(max_seqlen_q)]
+        if exact:
+            out[b:e] = torch.einsum("hts,shd->thd", torch.softmax(s64, dim=-1), v64).to(q.dtype)
+        else:
+            scores = torch.einsum("thd,shd->hts", qs, ks * scale)
+            if is_causal:
+                scores = scores + torch.triu(torch.full((n, n), -10000.0), 1).to(scores.dtype)
+            attention = torch.softmax(scores, dim=-1, dtype=vs.dtype)
+            out[b:e] = torch.einsum("hts,shd->thd", attention, vs)
+    return (out, lse) if return_lse else out

@@ -625,6 +625,89 @@ def test_context_attention_config4_full_size_sampled():
     assert_close(o2, vconst, rtol=1e-2, atol=1e-3, what="cfg4 full, constant V")
 
 
+# ----------------------------------------------------------------------------- variable-length flash attention
+# the reference's cases (diopi_configs.py:9854-9945): (q shape, key/value heads of the grouped case, cumulative lengths,
+# max_seqlen, is_causal, softmax_scale)
+FLASH_VARLEN_CASES = [
+    ((32, 32, 128), 4, [0, 32], 32, True, None),
+    ((64, 64, 128), 4, [0, 16, 48, 64], 32, True, 0.0883),
+    ((256, 16, 128), 2, [0, 32, 64, 128, 256], 128, False, None),
+    ((128, 8, 64), 2, [0, 16, 48, 64, 128], 64, True, 0.125),
+    ((512, 8, 64), 2, [0, 2, 7, 19, 32, 64, 96, 128, 256, 512], 256, False, None),
+    ((2784, 8, 64), 2, [0, 32, 96, 224, 2784], 2560, True, None),
+]
+
+
+def _flash_varlen_case(q, k, v, cu, max_seqlen, causal, scale, dt, what):
+    before = snapshot(q, k, v, cu)
+    out = F.flash_attention_varlen(q, k, v, cu, cu, None, max_seqlen, max_seqlen, 0, scale, causal, -1, -1)
+    lse = F.GLOBAL_STATE["flash_attention_varlen_softmax_lse"]
+    assert_unmodified(before, q, k, v, cu)
+    # the C interface carries the scale as a float (functions_ext.h:355-359): the oracle gets the value that arrives
+    scale = float(np.float32(scale if scale else 1.0 / math.sqrt(q.shape[-1])))
+    exact, lse64 = O.flash_attention_varlen(q.cpu(), k.cpu(), v.cpu(), cu.cpu(), cu.cpu(), None, max_seqlen, max_seqlen, 0, scale, causal, exact=True,
+                                            return_lse=True)
+    assert_close(out, exact, **TOL[dt], what=f"{what}: out vs float64")
+    if dt in (torch.float16, torch.bfloat16):
+        faithful = O.flash_attention_varlen(q.cpu(), k.cpu(), v.cpu(), cu.cpu(), cu.cpu(), None, max_seqlen, max_seqlen, 0, scale, causal)
+        # that composition rounds the scores and the probabilities to the 16-bit type, which moves single elements by
+        # more than the tolerance; the reference's own checker allows 1e-3 of the elements to miss (check_result.py:138-149)
+        assert_close(out, faithful, **TOL[dt], what=f"{what}: out vs the reference's composition", mismatch_ratio=1e-3)
+    # the log-sum-exp is a float32 output computed from fp32 scores of 16-bit inputs
+    assert_close(lse, lse64.float(), rtol=1e-4, atol=2e-3 if dt != torch.float32 else 1e-4, what=f"{what}: softmax_lse")
+    return out
+
+
+@pytest.mark.parametrize("case", range(len(FLASH_VARLEN_CASES)))
+@pytest.mark.parametrize("grouped", [False, True])
+def test_flash_attention_varlen_reference_cases(case, grouped):
+    shape, hkv_grouped, cu, max_seqlen, causal, scale = FLASH_VARLEN_CASES[case]
+    hkv = hkv_grouped if grouped else shape[1]
+    g = gen(800 + case)
+    for dt in (torch.float16, torch.bfloat16):
+        q = torch.randn(*shape, generator=g).to(dt).to(DEV)
+        k, v = (torch.randn(shape[0], hkv, shape[2], generator=g).to(dt).to(DEV) for _ in range(2))
+        cu_t = torch.tensor(cu, dtype=torch.int32, device=DEV)
+        _flash_varlen_case(q, k, v, cu_t, max_seqlen, causal, scale, dt, f"varlen case {case} grouped={grouped} {dt}")
+
+
+def test_flash_attention_varlen_long_sequences_and_int64_lengths():
+    # long enough for the 256-row query tiles, lengths that are no multiple of any tile size, full and causal attention
+    cu = [0, 1531, 2630, 2631]
+    g = gen(811)
+    for causal in (True, False):
+        q = (torch.randn(cu[-1], 8, 128, generator=g) * 0.5).half().to(DEV)
+        k, v = ((torch.randn(cu[-1], 2, 128, generator=g) * 0.5).half().to(DEV) for _ in range(2))
+        _flash_varlen_case(q, k, v, torch.tensor(cu, dtype=torch.int64, device=DEV), 1531, causal, None, torch.float16, f"long grouped causal={causal}")
+
+
+def test_flash_attention_varlen_matches_context_attention_and_other_dtypes():
+    w = W.cfg4(DEV, seed=4, scale=0.125)
+    cu = torch.cat((w["b_start_loc"], (w["b_start_loc"][-1:] + w["b_seq_len"][-1:]))).to(torch.int32)
+    ref = torch.zeros_like(w["q"])
+    F.context_attention(w["q"], w["k"], w["v"], ref, w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
+    out = F.flash_attention_varlen(w["q"], w["k"], w["v"], cu, cu, None, w["max_input_len"], w["max_input_len"], 0, None, True)
+    assert_close(out, ref, rtol=1e-3, atol=1e-3, what="causal multi-head varlen attention vs diopiContextAttentionInference")
+    g = gen(812)
+    for dt in (torch.float32, torch.float64):
+        q = torch.randn(40, 4, 48, generator=g, dtype=dt).to(DEV)
+        k, v = (torch.randn(40, 2, 48, generator=g, dtype=dt).to(DEV) for _ in range(2))
+        _flash_varlen_case(q, k, v, torch.tensor([0, 7, 7, 40], dtype=torch.int32, device=DEV), 33, False, 0.2, dt, f"{dt} with an empty sequence")
+
+
+def test_flash_attention_varlen_unsupported_modes_and_argument_errors():
+    q = torch.randn(8, 2, 128, device=DEV).half()
+    cu = torch.tensor([0, 8], dtype=torch.int32, device=DEV)
+    for kwargs in (dict(p_dropout=0.1), dict(window_size_left=4), dict(alibi_slopes=torch.ones(2, device=DEV))):
+        args = dict(alibi_slopes=None, p_dropout=0, window_size_left=-1)
+        args.update(kwargs)
+        with pytest.raises(rt.FunctionNotImplementedError):  # dropout, ALiBi and sliding windows answer with diopiNoImplement (13)
+            F.flash_attention_varlen(q, q, q, cu, cu, args["alibi_slopes"], 8, 8, args["p_dropout"], None, True, args["window_size_left"], -1)
+    with pytest.raises(rt.DiopiException):
+        F.flash_attention_varlen(q, q[:, :1].contiguous().repeat(1, 3, 1), q, cu, cu, None, 8, 8, 0, None, True)  # 2 query heads over 3 key heads
+    torch.cuda.synchronize()
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)

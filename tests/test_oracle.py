@@ -445,3 +445,67 @@ def test_context_attention_dtype_faithful_close_to_exact(dtype):
     O.context_attention(q, k, v, ex, bs, bl, exact=True)
     tol = 1e-2 if dtype == torch.float16 else 1e-5
     assert_close(out, ex, tol, tol, "reference composition vs float64")
+
+
+def test_flash_attention_varlen_causal_mha_is_context_attention():
+    g = rng(71)
+    cu = torch.tensor([0, 16, 48, 64], dtype=torch.int32)  # diopi_configs.py:9866, second case
+    q, k, v = (torch.randn(64, 4, 128, generator=g, dtype=torch.float64) for _ in range(3))
+    got = O.flash_attention_varlen(q, k, v, cu, cu, None, 32, 32, 0, None, True, -1, -1, exact=True)
+    want = torch.zeros_like(q)
+    O.context_attention(q, k, v, want, cu[:-1], cu[1:] - cu[:-1], 32, exact=True)
+    assert_close(got, want, 1e-12, 1e-12, "causal varlen attention vs the lightllm prefill statement")
+    # first token of every sequence: its own value row
+    for b in (0, 16, 48):
+        assert_close(got[b], v[b], 1e-14, 1e-15, "first token")
+
+
+def test_flash_attention_varlen_identical_keys_closed_form():
+    g = rng(72)
+    n, hq, hkv, d, scale = 9, 4, 2, 16, 0.3
+    q = torch.randn(n, hq, d, generator=g, dtype=torch.float64)
+    key = torch.randn(hkv, d, generator=g, dtype=torch.float64)
+    k = key.expand(n, hkv, d).contiguous()
+    v = torch.randn(n, hkv, d, generator=g, dtype=torch.float64)
+    cu = torch.tensor([0, n])
+    for causal in (True, False):
+        out, lse = O.flash_attention_varlen(q, k, v, cu, cu, None, n, n, 0, scale, causal, exact=True, return_lse=True)
+        for t in range(n):
+            cnt = t + 1 if causal else n
+            for h in range(hq):
+                assert_close(out[t, h], v[:cnt, h // 2].mean(0), 1e-13, 1e-13, "uniform weights -> mean of the visible values")
+                want = scale * float(q[t, h] @ key[h // 2]) + math.log(cnt)
+                assert abs(float(lse[0, h, t]) - want) < 1e-12
+
+
+def test_flash_attention_varlen_python_loops():
+    g = rng(73)
+    cu = [0, 2, 7, 19]  # ragged, as in diopi_configs.py:9866 (fifth case)
+    hq, hkv, d, scale = 4, 2, 8, 0.125
+    q = torch.randn(19, hq, d, generator=g, dtype=torch.float64)
+    k = torch.randn(19, hkv, d, generator=g, dtype=torch.float64)
+    v = torch.randn(19, hkv, d, generator=g, dtype=torch.float64)
+    for causal in (False, True):
+        out, lse = O.flash_attention_varlen(q, k, v, torch.tensor(cu), torch.tensor(cu), None, 12, 12, 0, scale, causal, exact=True, return_lse=True)
+        for i in range(3):
+            b, e = cu[i], cu[i + 1]
+            for t in range(b, e):
+                last = t if causal else e - 1
+                for h in range(hq):
+                    w = [math.exp(scale * sum(float(q[t, h, x]) * float(k[j, h // 2, x]) for x in range(d))) for j in range(b, last + 1)]
+                    tot = sum(w)
+                    for x in range(d):
+                        want = sum(w[j - b] * float(v[j, h // 2, x]) for j in range(b, last + 1)) / tot
+                        assert abs(float(out[t, h, x]) - want) < 1e-12
+                    assert abs(float(lse[i, h, t - b]) - math.log(tot)) < 1e-12
+        assert float(lse[0, :, 2:].abs().max()) == 0.0  # past the end of a short sequence
+
+
+def test_flash_attention_varlen_dtype_faithful_stays_near_exact():
+    g = rng(74)
+    cu = torch.tensor([0, 32, 64, 128, 256], dtype=torch.int32)  # diopi_configs.py:9866, third case (full attention)
+    q, k, v = (torch.randn(256, 16, 128, generator=g).half() for _ in range(3))
+    kk, vv = k[:, :2].contiguous(), v[:, :2].contiguous()  # the grouped case of 9929: 2 key/value heads
+    a = O.flash_attention_varlen(q, kk, vv, cu, cu, None, 128, 128, 0, None, False)
+    b = O.flash_attention_varlen(q, kk, vv, cu, cu, None, 128, 128, 0, None, False, exact=True)
+    assert_close(a.double(), b.double(), 1e-2, 1e-2, "fp16 composition vs float64")
