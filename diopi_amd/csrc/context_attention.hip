@@ -60,6 +60,7 @@ struct CtxArgs {
     int totalItems;    // H * tilesBound
     // general form only (diopiFlashAttentionVarLen); the lightllm operator leaves these at their defaults
     bool cumulative;   // bStartLoc holds batch + 1 cumulative lengths; bSeqLen is unused
+    int uniformLen;    // > 0: every sequence has this many rows and sequence i starts at row i * uniformLen (no index tensors)
     bool causal;
     int G;             // query heads per key/value head
     float scaleLog2;   // softmax scale * log2(e)
@@ -95,6 +96,11 @@ struct SeqInfo {
 
 __device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
     SeqInfo s;
+    if (a.uniformLen > 0) {
+        s.start = static_cast<int64_t>(i) * a.uniformLen;
+        s.len = a.uniformLen;
+        return s;
+    }
     s.start = loadIndex(a.bStartLoc, i, a.start64);
     s.len = a.cumulative ? loadIndex(a.bStartLoc, i + 1, a.start64) - s.start : loadIndex(a.bSeqLen, i, a.len64);
     if (s.start < 0 || s.start >= a.rows) s.len = 0;
@@ -625,6 +631,7 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     a.tilesBound = 0;
     a.totalItems = 0;
     a.cumulative = false;
+    a.uniformLen = 0;
     a.causal = true;
     a.G = 1;
     a.scaleLog2 = 0.f;
@@ -704,6 +711,7 @@ extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diop
     a.tilesBound = 0;
     a.totalItems = 0;
     a.cumulative = true;
+    a.uniformLen = 0;
     a.causal = is_causal;
     a.G = static_cast<int>(vQ.shape[1] / vK.shape[1]);
     const int D = static_cast<int>(vQ.shape[2]);
@@ -717,6 +725,80 @@ extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diop
     const diopiError_t err = dispatchAttention<true>(ctx, stream, vOut, vQ, vK, vV, a, D, scale);
     if (err != diopiDtypeNotSupported) return err;
     setLastError("diopiFlashAttentionVarLen: dtype %s is not supported", dtypeName(vQ.dtype));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}
+
+extern "C" diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                            diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                            diopiConstTensorHandle_t alibi_slopes, float p_dropout, float softmax_scale, bool is_causal,
+                                            int32_t window_size_left, int32_t window_size_right) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;  // only dropout draws random numbers
+    // the reference's statement covers neither of these (customized_test.py:463 "TODO: impl for alibi and sliding window")
+    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
+        setLastError("diopiFlashAttention: dropout, ALiBi slopes and sliding windows are not implemented");
+        return diopiNoImplement;
+    }
+    TensorView vOut, vQ, vK, vV, vLse;
+    ROCM_CALL(unwrap(attention_out, "attention_out", &vOut));
+    ROCM_CALL(unwrap(q, "q", &vQ));
+    ROCM_CALL(unwrap(k, "k", &vK));
+    ROCM_CALL(unwrap(v, "v", &vV));
+    ROCM_CALL(requireDeviceContiguous(vOut, "attention_out"));
+    ROCM_CALL(requireDeviceContiguous(vQ, "q"));
+    ROCM_CALL(requireDeviceContiguous(vK, "k"));
+    ROCM_CALL(requireDeviceContiguous(vV, "v"));
+    const bool haveLse = softmax_lse != nullptr;
+    if (haveLse) {
+        ROCM_CALL(unwrap(softmax_lse, "softmax_lse", &vLse));
+        ROCM_CALL(requireDeviceContiguous(vLse, "softmax_lse"));
+    }
+    ROCM_CHECK(vQ.ndim == 4 && vK.ndim == 4, "q and k must be [batch, seq_len, heads, head_dim], got ranks %d and %d", vQ.ndim, vK.ndim);
+    ROCM_CHECK(vOut.sameShape(vQ) && vV.sameShape(vK), "attention_out must have the shape of q, v the shape of k");
+    // like the reference's statement (customized_test.py:473-481: one seqlen for the mask), queries and keys are the same positions
+    ROCM_CHECK(vK.shape[0] == vQ.shape[0] && vK.shape[1] == vQ.shape[1] && vK.shape[3] == vQ.shape[3],
+               "q and k must have the same batch size, sequence length and head size");
+    ROCM_CHECK(vK.shape[2] > 0 && vQ.shape[2] % vK.shape[2] == 0, "the %lld query heads must be a multiple of the %lld key/value heads",
+               static_cast<long long>(vQ.shape[2]), static_cast<long long>(vK.shape[2]));
+    ROCM_CHECK(isFloatDtype(vQ.dtype) && vK.dtype == vQ.dtype && vV.dtype == vQ.dtype && vOut.dtype == vQ.dtype,
+               "q, k, v and attention_out must share one floating dtype (q is %s)", dtypeName(vQ.dtype));
+    ROCM_CHECK(vQ.shape[0] <= 65535 && vQ.shape[1] <= INT32_MAX && vQ.shape[2] <= INT32_MAX / 1024 && vQ.shape[3] <= 65535,
+               "batch / sequence length / head count / head size out of range");
+    if (haveLse) {
+        ROCM_CHECK(vLse.dtype == diopi_dtype_float32 && vLse.numel == vQ.shape[0] * vQ.shape[2] * vQ.shape[1],
+                   "softmax_lse must be float32 [batch, heads, seq_len] = [%lld, %lld, %lld]", static_cast<long long>(vQ.shape[0]),
+                   static_cast<long long>(vQ.shape[2]), static_cast<long long>(vQ.shape[1]));
+    }
+    if (vQ.numel == 0) return diopiSuccess;
+
+    CtxArgs a;
+    a.bStartLoc = nullptr;
+    a.bSeqLen = nullptr;
+    a.start64 = false;
+    a.len64 = false;
+    a.batch = static_cast<int>(vQ.shape[0]);
+    a.H = static_cast<int>(vQ.shape[2]);
+    a.rows = vQ.shape[0] * vQ.shape[1];
+    a.tilesBound = 0;
+    a.totalItems = 0;
+    a.cumulative = false;
+    a.uniformLen = static_cast<int>(vQ.shape[1]);
+    a.causal = is_causal;
+    a.G = static_cast<int>(vQ.shape[2] / vK.shape[2]);
+    const int D = static_cast<int>(vQ.shape[3]);
+    const double scale = softmax_scale != 0.f ? static_cast<double>(softmax_scale) : 1.0 / std::sqrt(static_cast<double>(D));
+    a.scaleLog2 = static_cast<float>(scale * 1.4426950408889634);
+    a.lse = haveLse ? static_cast<float*>(vLse.data) : nullptr;
+    a.lseStride = static_cast<int>(vQ.shape[1]);
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    // the kernels see the packed [batch * seq_len, heads, head_dim] view
+    TensorView pq = vQ, pk = vK, pv = vV, po = vOut;
+    const diopiError_t err = dispatchAttention<true>(ctx, stream, po, pq, pk, pv, a, D, scale);
+    if (err != diopiDtypeNotSupported) return err;
+    setLastError("diopiFlashAttention: dtype %s is not supported", dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
     ROCM_ENTRY_END
 }

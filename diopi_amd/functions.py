@@ -199,3 +199,20 @@ def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu
     check_returncode(ret, "diopiFlashAttentionVarLen")
     GLOBAL_STATE["flash_attention_varlen_softmax_lse"] = lse
     return out
+
+
+def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alibi_slopes, p_dropout: float, softmax_scale, is_causal: bool,
+                    window_size_left: int = -1, window_size_right: int = -1, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py flash_attention of the reference: allocates out and softmax_lse [batch, heads, seq_len] (kept in
+    GLOBAL_STATE["flash_attention_softmax_lse"]), replaces a missing scale by 1/sqrt(head_dim), returns out."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(q)
+    lse = torch.zeros(q.shape[0], q.shape[2], q.shape[1], dtype=torch.float32, device=q.device)
+    scale = 1.0 / math.sqrt(q.shape[-1]) if not softmax_scale else float(softmax_scale)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, lse, q, k, v, alibi_slopes)
+        ret = rt.libs().impl.diopiFlashAttention(ctx.handle, h[0], h[1], None, h[2], h[3], h[4], h[5], float(p_dropout), scale, bool(is_causal),
+                                                 int(window_size_left), int(window_size_right))
+    check_returncode(ret, "diopiFlashAttention")
+    GLOBAL_STATE["flash_attention_softmax_lse"] = lse
+    return out

@@ -146,6 +146,7 @@ class _Libs:
         impl.diopiContextAttentionInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
         impl.diopiFlashAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, ctypes.c_float, ctypes.c_float, ctypes.c_bool,
                                                    i32, i32]
+        impl.diopiFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_float, ctypes.c_float, ctypes.c_bool, i32, i32]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
@@ -163,6 +164,7 @@ OPERATOR_SYMBOLS = (
     "diopiTokenSoftmaxReduceVInference",
     "diopiContextAttentionInference",
     "diopiFlashAttentionVarLen",
+    "diopiFlashAttention",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

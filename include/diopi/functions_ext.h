@@ -157,6 +157,17 @@ DIOPI_API diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diopi
                                                  int32_t max_seqlen_q, int32_t max_seqlen_kv, float p_dropout, float softmax_scale, bool is_causal,
                                                  int32_t window_size_left, int32_t window_size_right);
 
+/*
+ * Flash attention on padded batches, forward.
+ * reference: functions_ext.h:209-212 (Python statement customized_test.py:462-485).
+ * q [batch, seq_len, Hq, D]; k, v [batch, seq_len, Hkv, D] (same seq_len, as in the reference's statement), Hq a
+ * multiple of Hkv; softmax_lse [batch, Hq, seq_len] float32, may be null.  Everything else as diopiFlashAttentionVarLen.
+ */
+DIOPI_API diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                           diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                           diopiConstTensorHandle_t alibi_slopes, float p_dropout, float softmax_scale, bool is_causal,
+                                           int32_t window_size_left, int32_t window_size_right);
+
 #if defined(__cplusplus)
 }
 #endif

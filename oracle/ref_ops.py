@@ -22,6 +22,7 @@ destindex_copy_kv            functions_lightllm.cpp:18-26; customized_test.py:69
 token_attention              functions_lightllm.cpp:53-80; customized_test.py:698-713
 token_softmax_reducev        functions_lightllm.cpp:82-107; customized_test.py:715-733
 context_attention            functions_lightllm.cpp:109-147; customized_test.py:8-33, 735-749
+flash_attention              customized_test.py:462-485 (declaration functions_ext.h:209-212)
 flash_attention_varlen       customized_test.py:525-588 with multi_head_attention_inside, 36-57 (the torch
                              implementation calls the flash-attn library; declaration functions_ext.h:355-359)
 ===========================  =====================================================================
@@ -61,6 +62,8 @@ How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"
                        brute force with explicit Python loops
   token_softmax_reducev  constant logits -> mean of the gathered rows, one dominant logit -> that row,
                        L=1 -> the row bit for bit, float64 brute force
+  flash_attention      agreement with flash_attention_varlen on the flattened batch (two restatements written from
+                       different reference functions), explicit Python loops
   flash_attention_varlen  causal multi-head case = context_attention on the same tokens, identical keys ->
                        mean of the visible values and lse = scale*q.k + ln(count), explicit Python loops for
                        full attention, grouped heads, a custom scale and the log-sum-exp
@@ -322,4 +325,29 @@ def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu
                 scores = scores + torch.triu(torch.full((n, n), -10000.0), 1).to(scores.dtype)
             attention = torch.softmax(scores, dim=-1, dtype=vs.dtype)
             out[b:e] = torch.einsum("hts,shd->thd", attention, vs)
+    return (out, lse) if return_lse else out
+
+
+def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alibi_slopes, p_dropout: float, softmax_scale, is_causal: bool,
+                    window_size_left: int = -1, window_size_right: int = -1, exact: bool = False, return_lse: bool = False):
+    """customized_test.py:462-485: q [b, t, h, d], k/v [b, s, hkv, d] with hkv heads repeated g times; scores = einsum of q
+    with k * scale (in the tensor dtype), -inf above the diagonal if causal, softmax with dtype=v.dtype, einsum with v.
+    exact=True: float64 throughout, rounded once.  return_lse: also the float64 log-sum-exp [b, h, t]."""
+    assert alibi_slopes is None and p_dropout == 0 and window_size_left < 0 and window_size_right < 0, "not covered by the reference's statement"
+    g = q.shape[2] // k.shape[2]
+    if g > 1:
+        k, v = k.repeat_interleave(g, dim=2), v.repeat_interleave(g, dim=2)
+    seqlen = q.shape[1]
+    scale = softmax_scale or 1.0 / math.sqrt(q.shape[-1])
+    s64 = torch.einsum("bthd,bshd->bhts", q.double(), k.double()) * scale
+    if is_causal:
+        s64 = s64 + torch.triu(torch.full((seqlen, seqlen), float("-inf"), dtype=torch.float64), 1)
+    lse = torch.logsumexp(s64, dim=-1)
+    if exact:
+        out = torch.einsum("bhts,bshd->bthd", torch.softmax(s64, dim=-1), v.double()).to(q.dtype)
+    else:
+        scores = torch.einsum("bthd,bshd->bhts", q, k * scale)
+        if is_causal:
+            scores = scores + torch.triu(torch.full((seqlen, seqlen), float("-inf")), 1).to(dtype=scores.dtype)
+        out = torch.einsum("bhts,bshd->bthd", torch.softmax(scores, dim=-1, dtype=v.dtype), v)
     return (out, lse) if return_lse else out

@@ -37,6 +37,8 @@ diopiError_t diopiContextAttentionInference(diopiContextHandle_t, diopiTensorHan
 diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiGeneratorHandle_t, diopiConstTensorHandle_t,
                                        diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
                                        diopiConstTensorHandle_t, int32_t, int32_t, float, float, bool, int32_t, int32_t);
+diopiError_t diopiFlashAttention(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiGeneratorHandle_t, diopiConstTensorHandle_t,
+                                 diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, float, float, bool, int32_t, int32_t);
 // the callbacks the library imports
 diopiError_t diopiGetTensorShape(diopiConstTensorHandle_t, diopiSize_t*);
 diopiError_t diopiGetStream(diopiContextHandle_t, diopiStreamHandle_t*);

@@ -708,6 +708,34 @@ def test_flash_attention_varlen_unsupported_modes_and_argument_errors():
     torch.cuda.synchronize()
 
 
+# the reference's cases for the padded layout (diopi_configs.py:9770-9852): (q shape, key/value heads, is_causal, softmax_scale)
+FLASH_CASES = [
+    ((1, 64, 64, 128), 64, True, 0.0883), ((1, 256, 16, 128), 16, False, None), ((1, 64, 32, 128), 32, True, 0.125), ((1, 16, 8, 64), 8, True, 0.125),
+    ((2, 64, 64, 128), 8, True, 0.0883), ((1, 256, 32, 128), 8, False, None), ((8, 32, 32, 128), 8, True, 0.125),
+]
+
+
+@pytest.mark.parametrize("case", range(len(FLASH_CASES)))
+def test_flash_attention_reference_cases(case):
+    shape, hkv, causal, scale = FLASH_CASES[case]
+    g = gen(900 + case)
+    for dt in (torch.float16, torch.bfloat16):
+        q = torch.randn(*shape, generator=g).to(dt).to(DEV)
+        k, v = (torch.randn(shape[0], shape[1], hkv, shape[3], generator=g).to(dt).to(DEV) for _ in range(2))
+        before = snapshot(q, k, v)
+        out = F.flash_attention(q, k, v, None, 0, scale, causal, -1, -1)
+        lse = F.GLOBAL_STATE["flash_attention_softmax_lse"]
+        assert_unmodified(before, q, k, v)
+        sc = float(np.float32(scale if scale else 1.0 / math.sqrt(shape[3])))
+        exact, lse64 = O.flash_attention(q.cpu(), k.cpu(), v.cpu(), None, 0, sc, causal, exact=True, return_lse=True)
+        assert_close(out, exact, **TOL[dt], what=f"padded case {case} {dt}: out vs float64")
+        faithful = O.flash_attention(q.cpu(), k.cpu(), v.cpu(), None, 0, sc, causal)
+        assert_close(out, faithful, **TOL[dt], what=f"padded case {case} {dt}: out vs the reference's composition", mismatch_ratio=1e-3)
+        assert_close(lse, lse64.float(), rtol=1e-4, atol=2e-3, what=f"padded case {case} {dt}: softmax_lse")
+    with pytest.raises(rt.FunctionNotImplementedError):
+        F.flash_attention(q, k, v, None, 0.5, scale, causal, -1, -1)
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)

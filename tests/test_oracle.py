@@ -509,3 +509,26 @@ def test_flash_attention_varlen_dtype_faithful_stays_near_exact():
     a = O.flash_attention_varlen(q, kk, vv, cu, cu, None, 128, 128, 0, None, False)
     b = O.flash_attention_varlen(q, kk, vv, cu, cu, None, 128, 128, 0, None, False, exact=True)
     assert_close(a.double(), b.double(), 1e-2, 1e-2, "fp16 composition vs float64")
+
+
+def test_flash_attention_agrees_with_varlen_and_loops():
+    g = rng(75)
+    b, t, hq, hkv, d, scale = 3, 5, 4, 2, 8, 0.2
+    q = torch.randn(b, t, hq, d, generator=g, dtype=torch.float64)
+    k = torch.randn(b, t, hkv, d, generator=g, dtype=torch.float64)
+    v = torch.randn(b, t, hkv, d, generator=g, dtype=torch.float64)
+    cu = torch.arange(0, (b + 1) * t, t)
+    for causal in (True, False):
+        out, lse = O.flash_attention(q, k, v, None, 0, scale, causal, exact=True, return_lse=True)
+        o2, l2 = O.flash_attention_varlen(q.reshape(b * t, hq, d), k.reshape(b * t, hkv, d), v.reshape(b * t, hkv, d), cu, cu, None, t, t, 0, scale, causal,
+                                          exact=True, return_lse=True)
+        assert_close(out.reshape(b * t, hq, d), o2, 1e-12, 1e-12, "padded vs variable-length restatement")
+        assert_close(lse, l2, 1e-12, 1e-12, "log-sum-exp")
+        for bi in range(b):
+            for ti in range(t):
+                last = ti if causal else t - 1
+                for h in range(hq):
+                    w = [math.exp(scale * float(q[bi, ti, h] @ k[bi, j, h // 2])) for j in range(last + 1)]
+                    want = sum(w[j] * v[bi, j, h // 2] for j in range(last + 1)) / sum(w)
+                    assert_close(out[bi, ti, h], want, 1e-12, 1e-12, "loops")
+                    assert abs(float(lse[bi, h, ti]) - math.log(sum(w))) < 1e-12
