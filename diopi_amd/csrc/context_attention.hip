@@ -647,20 +647,13 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     ROCM_ENTRY_END
 }
 
-extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
-                                                  diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
-                                                  diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_kv, diopiConstTensorHandle_t alibi_slopes,
-                                                  int32_t max_seqlen_q, int32_t max_seqlen_kv, float p_dropout, float softmax_scale, bool is_causal,
-                                                  int32_t window_size_left, int32_t window_size_right) {
-    ROCM_ENTRY_BEGIN
-    using namespace rocm;
-    (void)gen;            // only dropout draws random numbers
-    (void)max_seqlen_kv;  // lengths come from the cumulative tensors
-    // the reference's statement covers neither of these (customized_test.py:540 "TODO: impl for alibi and sliding window")
-    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
-        setLastError("diopiFlashAttentionVarLen: dropout, ALiBi slopes and sliding windows are not implemented");
-        return diopiNoImplement;
-    }
+namespace rocm {
+namespace {
+
+// Variable-length attention behind diopiFlashAttentionVarLen and diopiMultiHeadAttentionVarLen.
+diopiError_t attentionVarLen(diopiContextHandle_t ctx, const char* opName, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                             diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t cum_seq_q,
+                             diopiConstTensorHandle_t cum_seq_kv, int64_t max_seqlen_q, double softmax_scale, bool is_causal) {
     TensorView vOut, vQ, vK, vV, vCuQ, vCuK, vLse;
     ROCM_CALL(unwrap(attention_out, "attention_out", &vOut));
     ROCM_CALL(unwrap(q, "q", &vQ));
@@ -691,12 +684,12 @@ extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diop
                    vCuK.dtype == vCuQ.dtype,
                "cum_seq_q and cum_seq_kv must be 1-D int32 or int64 tensors of batch + 1 entries");
     ROCM_CHECK(vCuQ.shape[0] - 1 <= 65535 && vQ.shape[1] <= INT32_MAX / 1024 && vQ.shape[2] <= 65535, "batch / head count / head size out of range");
-    ROCM_CHECK(max_seqlen_q >= 0, "max_seqlen_q must not be negative");
+    ROCM_CHECK(max_seqlen_q >= 0 && max_seqlen_q <= INT32_MAX, "max_seqlen_q out of range");
     const int64_t batch = vCuQ.shape[0] - 1;
     if (haveLse) {
         ROCM_CHECK(vLse.dtype == diopi_dtype_float32 && vLse.numel == batch * vQ.shape[1] * static_cast<int64_t>(max_seqlen_q),
-                   "softmax_lse must be float32 [batch, heads, max_seqlen_q] = [%lld, %lld, %d]", static_cast<long long>(batch),
-                   static_cast<long long>(vQ.shape[1]), max_seqlen_q);
+                   "softmax_lse must be float32 [batch, heads, max_seqlen_q] = [%lld, %lld, %lld]", static_cast<long long>(batch),
+                   static_cast<long long>(vQ.shape[1]), static_cast<long long>(max_seqlen_q));
     }
     if (vQ.numel == 0 || batch == 0) return diopiSuccess;
 
@@ -716,31 +709,21 @@ extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diop
     a.G = static_cast<int>(vQ.shape[1] / vK.shape[1]);
     const int D = static_cast<int>(vQ.shape[2]);
     // the Python layer passes 1/sqrt(head_dim) for "None" (diopi_functions.py:7564-7566); zero means the same here
-    const double scale = softmax_scale != 0.f ? static_cast<double>(softmax_scale) : 1.0 / std::sqrt(static_cast<double>(D));
+    const double scale = softmax_scale != 0.0 ? softmax_scale : 1.0 / std::sqrt(static_cast<double>(D));
     a.scaleLog2 = static_cast<float>(scale * 1.4426950408889634);
     a.lse = haveLse ? static_cast<float*>(vLse.data) : nullptr;
-    a.lseStride = max_seqlen_q;
+    a.lseStride = static_cast<int>(max_seqlen_q);
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
     const diopiError_t err = dispatchAttention<true>(ctx, stream, vOut, vQ, vK, vV, a, D, scale);
     if (err != diopiDtypeNotSupported) return err;
-    setLastError("diopiFlashAttentionVarLen: dtype %s is not supported", dtypeName(vQ.dtype));
+    setLastError("%s: dtype %s is not supported", opName, dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
-    ROCM_ENTRY_END
 }
 
-extern "C" diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
-                                            diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
-                                            diopiConstTensorHandle_t alibi_slopes, float p_dropout, float softmax_scale, bool is_causal,
-                                            int32_t window_size_left, int32_t window_size_right) {
-    ROCM_ENTRY_BEGIN
-    using namespace rocm;
-    (void)gen;  // only dropout draws random numbers
-    // the reference's statement covers neither of these (customized_test.py:463 "TODO: impl for alibi and sliding window")
-    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
-        setLastError("diopiFlashAttention: dropout, ALiBi slopes and sliding windows are not implemented");
-        return diopiNoImplement;
-    }
+// Attention on padded batches behind diopiFlashAttention and diopiMultiHeadAttention.
+diopiError_t attentionPadded(diopiContextHandle_t ctx, const char* opName, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                             diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, double softmax_scale, bool is_causal) {
     TensorView vOut, vQ, vK, vV, vLse;
     ROCM_CALL(unwrap(attention_out, "attention_out", &vOut));
     ROCM_CALL(unwrap(q, "q", &vQ));
@@ -788,7 +771,7 @@ extern "C" diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTenso
     a.causal = is_causal;
     a.G = static_cast<int>(vQ.shape[2] / vK.shape[2]);
     const int D = static_cast<int>(vQ.shape[3]);
-    const double scale = softmax_scale != 0.f ? static_cast<double>(softmax_scale) : 1.0 / std::sqrt(static_cast<double>(D));
+    const double scale = softmax_scale != 0.0 ? softmax_scale : 1.0 / std::sqrt(static_cast<double>(D));
     a.scaleLog2 = static_cast<float>(scale * 1.4426950408889634);
     a.lse = haveLse ? static_cast<float*>(vLse.data) : nullptr;
     a.lseStride = static_cast<int>(vQ.shape[1]);
@@ -798,7 +781,79 @@ extern "C" diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTenso
     TensorView pq = vQ, pk = vK, pv = vV, po = vOut;
     const diopiError_t err = dispatchAttention<true>(ctx, stream, po, pq, pk, pv, a, D, scale);
     if (err != diopiDtypeNotSupported) return err;
-    setLastError("diopiFlashAttention: dtype %s is not supported", dtypeName(vQ.dtype));
+    setLastError("%s: dtype %s is not supported", opName, dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
+}
+
+}  // namespace
+}  // namespace rocm
+
+extern "C" diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                                  diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                                  diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_kv, diopiConstTensorHandle_t alibi_slopes,
+                                                  int32_t max_seqlen_q, int32_t max_seqlen_kv, float p_dropout, float softmax_scale, bool is_causal,
+                                                  int32_t window_size_left, int32_t window_size_right) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;            // only dropout draws random numbers
+    (void)max_seqlen_kv;  // lengths come from the cumulative tensors
+    // the reference's statement covers neither of these (customized_test.py:540 "TODO: impl for alibi and sliding window")
+    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
+        setLastError("diopiFlashAttentionVarLen: dropout, ALiBi slopes and sliding windows are not implemented");
+        return diopiNoImplement;
+    }
+    return attentionVarLen(ctx, "diopiFlashAttentionVarLen", attention_out, softmax_lse, q, k, v, cum_seq_q, cum_seq_kv, max_seqlen_q, softmax_scale,
+                           is_causal);
+    ROCM_ENTRY_END
+}
+
+extern "C" diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t attention_out, diopiTensorHandle_t softmax_lse,
+                                            diopiGeneratorHandle_t gen, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                            diopiConstTensorHandle_t alibi_slopes, float p_dropout, float softmax_scale, bool is_causal,
+                                            int32_t window_size_left, int32_t window_size_right) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;  // only dropout draws random numbers
+    // the reference's statement covers neither of these (customized_test.py:463 "TODO: impl for alibi and sliding window")
+    if (p_dropout != 0.f || alibi_slopes != nullptr || window_size_left >= 0 || window_size_right >= 0) {
+        setLastError("diopiFlashAttention: dropout, ALiBi slopes and sliding windows are not implemented");
+        return diopiNoImplement;
+    }
+    return attentionPadded(ctx, "diopiFlashAttention", attention_out, softmax_lse, q, k, v, softmax_scale, is_causal);
+    ROCM_ENTRY_END
+}
+
+// The two older names of the same operators (proto/include/diopi/functions_ext.h:93-95 and 150-153, "deprecated: use
+// diopiFlashAttention / diopiFlashAttentionVarLen instead"; Python statements customized_test.py:416-460).  No grouped
+// heads in their statement, but nothing here depends on that.  The debug mask only exists with dropout.
+extern "C" diopiError_t diopiMultiHeadAttention(diopiContextHandle_t ctx, diopiTensorHandle_t q, diopiTensorHandle_t k, diopiTensorHandle_t v, double dropout_p,
+                                                bool is_causal, bool return_debug_mask, double scale, diopiTensorHandle_t out, diopiTensorHandle_t softmax_lse,
+                                                diopiGeneratorHandle_t gen, diopiTensorHandle_t debug_attn_mask) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;
+    (void)debug_attn_mask;
+    if (dropout_p != 0.0 || return_debug_mask) {
+        setLastError("diopiMultiHeadAttention: dropout and its debug mask are not implemented");
+        return diopiNoImplement;
+    }
+    return attentionPadded(ctx, "diopiMultiHeadAttention", out, softmax_lse, q, k, v, scale, is_causal);
+    ROCM_ENTRY_END
+}
+
+extern "C" diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t q, diopiTensorHandle_t k, diopiTensorHandle_t v,
+                                                      diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_k, int64_t max_q, int64_t max_k,
+                                                      double dropout_p, bool is_causal, bool return_debug_mask, double scale, diopiTensorHandle_t out,
+                                                      diopiTensorHandle_t softmax_lse, diopiGeneratorHandle_t gen, diopiTensorHandle_t debug_attn_mask) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)gen;
+    (void)debug_attn_mask;
+    (void)max_k;
+    if (dropout_p != 0.0 || return_debug_mask) {
+        setLastError("diopiMultiHeadAttentionVarLen: dropout and its debug mask are not implemented");
+        return diopiNoImplement;
+    }
+    return attentionVarLen(ctx, "diopiMultiHeadAttentionVarLen", out, softmax_lse, q, k, v, cum_seq_q, cum_seq_k, max_q, scale, is_causal);
     ROCM_ENTRY_END
 }

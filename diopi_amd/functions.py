@@ -216,3 +216,35 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alibi_slo
     check_returncode(ret, "diopiFlashAttention")
     GLOBAL_STATE["flash_attention_softmax_lse"] = lse
     return out
+
+
+def multihead_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, dropout_p: float, is_causal: bool, return_debug_mask: bool, scale,
+                        ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py:7112-7149 of the reference (softmax_lse kept in GLOBAL_STATE["multihead_attention_softmax_lse"])."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(q)
+    lse = torch.zeros(q.shape[0], q.shape[2], q.shape[1], dtype=torch.float32, device=q.device)
+    softmax_scale = 1.0 / math.sqrt(q.shape[-1]) if not scale else float(scale)
+    with _on_stream(ctx, out):
+        keep, h = _handles(q, k, v, out, lse)
+        ret = rt.libs().impl.diopiMultiHeadAttention(ctx.handle, h[0], h[1], h[2], float(dropout_p), bool(is_causal), bool(return_debug_mask), softmax_scale,
+                                                     h[3], h[4], None, None)
+    check_returncode(ret, "diopiMultiHeadAttention")
+    GLOBAL_STATE["multihead_attention_softmax_lse"] = lse
+    return out
+
+
+def multihead_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor, max_seqlen: int, dropout_p: float,
+                               is_causal: bool, return_debug_mask: bool, scale, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py:7195-7250 of the reference (softmax_lse kept in GLOBAL_STATE["multihead_attention_varlen_softmax_lse"])."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(q)
+    lse = torch.zeros(cu_seqlens.numel() - 1, q.shape[1], int(max_seqlen), dtype=torch.float32, device=q.device)
+    softmax_scale = 1.0 / math.sqrt(q.shape[-1]) if not scale else float(scale)
+    with _on_stream(ctx, out):
+        keep, h = _handles(q, k, v, cu_seqlens, out, lse)
+        ret = rt.libs().impl.diopiMultiHeadAttentionVarLen(ctx.handle, h[0], h[1], h[2], h[3], h[3], int(max_seqlen), int(max_seqlen), float(dropout_p),
+                                                           bool(is_causal), bool(return_debug_mask), softmax_scale, h[4], h[5], None, None)
+    check_returncode(ret, "diopiMultiHeadAttentionVarLen")
+    GLOBAL_STATE["multihead_attention_varlen_softmax_lse"] = lse
+    return out

@@ -147,6 +147,9 @@ class _Libs:
         impl.diopiFlashAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, ctypes.c_float, ctypes.c_float, ctypes.c_bool,
                                                    i32, i32]
         impl.diopiFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_float, ctypes.c_float, ctypes.c_bool, i32, i32]
+        i64, dbl = ctypes.c_int64, ctypes.c_double
+        impl.diopiMultiHeadAttention.argtypes = [vp, vp, vp, vp, dbl, ctypes.c_bool, ctypes.c_bool, dbl, vp, vp, vp, vp]
+        impl.diopiMultiHeadAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ctypes.c_bool, ctypes.c_bool, dbl, vp, vp, vp, vp]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
@@ -165,6 +168,8 @@ OPERATOR_SYMBOLS = (
     "diopiContextAttentionInference",
     "diopiFlashAttentionVarLen",
     "diopiFlashAttention",
+    "diopiMultiHeadAttention",
+    "diopiMultiHeadAttentionVarLen",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

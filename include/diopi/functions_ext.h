@@ -168,6 +168,19 @@ DIOPI_API diopiError_t diopiFlashAttention(diopiContextHandle_t ctx, diopiTensor
                                            diopiConstTensorHandle_t alibi_slopes, float p_dropout, float softmax_scale, bool is_causal,
                                            int32_t window_size_left, int32_t window_size_right);
 
+/*
+ * The older names of the two operators above (reference: functions_ext.h:93-95 and 150-153, marked deprecated there;
+ * Python statements customized_test.py:416-460).  q, k, v are not modified.  dropout_p != 0 or return_debug_mask answer
+ * 13; gen and debug_attn_mask are not used.  scale == 0 means 1/sqrt(D).
+ */
+DIOPI_API diopiError_t diopiMultiHeadAttention(diopiContextHandle_t ctx, diopiTensorHandle_t q, diopiTensorHandle_t k, diopiTensorHandle_t v, double dropout_p,
+                                               bool is_causal, bool return_debug_mask, double scale, diopiTensorHandle_t out, diopiTensorHandle_t softmax_lse,
+                                               diopiGeneratorHandle_t gen, diopiTensorHandle_t debug_attn_mask);
+DIOPI_API diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t ctx, diopiTensorHandle_t q, diopiTensorHandle_t k, diopiTensorHandle_t v,
+                                                     diopiConstTensorHandle_t cum_seq_q, diopiConstTensorHandle_t cum_seq_k, int64_t max_q, int64_t max_k,
+                                                     double dropout_p, bool is_causal, bool return_debug_mask, double scale, diopiTensorHandle_t out,
+                                                     diopiTensorHandle_t softmax_lse, diopiGeneratorHandle_t gen, diopiTensorHandle_t debug_attn_mask);
+
 #if defined(__cplusplus)
 }
 #endif

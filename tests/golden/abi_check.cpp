@@ -39,6 +39,11 @@ diopiError_t diopiFlashAttentionVarLen(diopiContextHandle_t, diopiTensorHandle_t
                                        diopiConstTensorHandle_t, int32_t, int32_t, float, float, bool, int32_t, int32_t);
 diopiError_t diopiFlashAttention(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiGeneratorHandle_t, diopiConstTensorHandle_t,
                                  diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, float, float, bool, int32_t, int32_t);
+diopiError_t diopiMultiHeadAttention(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, double, bool, bool, double,
+                                     diopiTensorHandle_t, diopiTensorHandle_t, diopiGeneratorHandle_t, diopiTensorHandle_t);
+diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t,
+                                           diopiConstTensorHandle_t, int64_t, int64_t, double, bool, bool, double, diopiTensorHandle_t, diopiTensorHandle_t,
+                                           diopiGeneratorHandle_t, diopiTensorHandle_t);
 // the callbacks the library imports
 diopiError_t diopiGetTensorShape(diopiConstTensorHandle_t, diopiSize_t*);
 diopiError_t diopiGetStream(diopiContextHandle_t, diopiStreamHandle_t*);

@@ -736,6 +736,30 @@ def test_flash_attention_reference_cases(case):
         F.flash_attention(q, k, v, None, 0.5, scale, causal, -1, -1)
 
 
+def test_multihead_attention_older_names():
+    # the reference's cases for the deprecated names (diopi_configs.py, multihead_attention / multihead_attention_varlen):
+    # the same statement (multi_head_attention_inside) as the flash-attention operators, so the same oracle serves
+    g = gen(950)
+    q, k, v = (torch.randn(2, 128, 8, 128, generator=g).half().to(DEV) for _ in range(3))
+    for causal, scale in ((True, None), (False, 0.1)):
+        out = F.multihead_attention(q, k, v, 0, causal, False, scale)
+        lse = F.GLOBAL_STATE["multihead_attention_softmax_lse"]
+        exact, lse64 = O.flash_attention(q.cpu(), k.cpu(), v.cpu(), None, 0, scale, causal, exact=True, return_lse=True)
+        assert_close(out, exact, **TOL[torch.float16], what="multihead_attention")
+        assert_close(lse, lse64.float(), rtol=1e-4, atol=2e-3, what="multihead_attention softmax_lse")
+    cu = torch.tensor([0, 37, 37, 200, 256], dtype=torch.int64, device=DEV)
+    qp, kp, vp = (t.reshape(256, 8, 128) for t in (q, k, v))
+    out = F.multihead_attention_varlen(qp, kp, vp, cu, 163, 0, True, False, None)
+    lse = F.GLOBAL_STATE["multihead_attention_varlen_softmax_lse"]
+    exact, lse64 = O.flash_attention_varlen(qp.cpu(), kp.cpu(), vp.cpu(), cu.cpu(), cu.cpu(), None, 163, 163, 0, None, True, exact=True, return_lse=True)
+    assert_close(out, exact, **TOL[torch.float16], what="multihead_attention_varlen")
+    assert_close(lse, lse64.float(), rtol=1e-4, atol=2e-3, what="multihead_attention_varlen softmax_lse")
+    with pytest.raises(rt.FunctionNotImplementedError):
+        F.multihead_attention(q, k, v, 0.1, True, False, None)
+    with pytest.raises(rt.FunctionNotImplementedError):
+        F.multihead_attention_varlen(qp, kp, vp, cu, 163, 0, True, True, None)
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
