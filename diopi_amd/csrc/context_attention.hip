@@ -42,9 +42,8 @@ namespace {
 constexpr int kBMMin = 128;  // smallest query tile of a work-group (bounds of the planning step are sized for it)
 constexpr int kBN = 64;    // key rows per tile
 constexpr int kHD = 128;   // head size of the MFMA kernel
-constexpr int kLD = kHD + 8;  // LDS row pitch in elements (272 bytes: 16-byte aligned, conflict-free 128-bit reads)
-constexpr int kVP = kBN + 8;   // row pitch of the transposed V tile in elements (144 bytes)
-constexpr int kStageElems = kBN * kLD + kHD * kVP;  // one staging buffer (K tile + transposed V tile), in elements
+constexpr int kLD = kHD + 8;  // row pitch of the output tile in LDS, in elements (272 bytes: 16-byte aligned)
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 constexpr int kNumXcd = 8;
 constexpr float kLazyLog2 = 8.0f;  // how far (in powers of two) the softmax reference maximum may lag behind
 
@@ -87,6 +86,17 @@ union FragBits {
     Frag f;
     __device__ FragBits() {}
 };
+
+// One 16-byte load per lane from a raw buffer straight into LDS: lane l's packet lands at ldsAddr + 16 l.  The LDS
+// base travels in M0 (wave-uniform).  Written as assembly so that the compiler does not order later LDS reads of
+// other addresses behind the load; the issuer must call waitLdsLoads() before the barrier that publishes the data.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void loadToLds16(u32x4 rsrc, uint32_t ldsAddr, int byteOffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(ldsAddr), "v"(byteOffset), "s"(rsrc) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ void waitLdsLoads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Sequence geometry with every value forced inside the tensors.
 struct SeqInfo {
@@ -163,8 +173,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     using Ops = Mfma32<T>;
     using Frag = typename Ops::Frag;
     constexpr int BM = NWV * 32;  // query rows per work-group: each of the NWV waves owns 32 of them
-    constexpr int kThreads = NWV * kWave;
-    // two staging buffers of (K tile [key][dim] row-major, V tile transposed [dim row][key position], see below)
+    // two staging buffers of (K tile, V tile), both [key][dim] row-major with swizzled 16-byte packets, see below
     extern __shared__ __attribute__((aligned(16))) unsigned char dynSmem[];
     T* smem = reinterpret_cast<T*>(dynSmem);
 
@@ -218,105 +227,83 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     const int waveRowLo = m0 + wave * 32;
     const int waveRowHi = waveRowLo + 31;
 
-    // ---- tile staging ----
-    // K: thread -> 16-byte packet ldC of rows ldR, ldR+16, ldR+32, ldR+48, stored as they are.
-    // V: stored transposed, sVt[row(dim)][position(key)], so that the A operand of the second product (8 keys of one
-    //    dim) is one 16-byte read.  A thread takes packet ldC (dims 8*ldC .. +7) of two adjacent keys, interleaves
-    //    them with byte permutes and writes one dword (key pair) per dim.  The row of dim 8*c + e is 16*e + c and
-    //    the keys of a 16-key group sit in the order (0-3, 8-11, 4-7, 12-15): with the 144-byte row pitch this makes
-    //    both the dword writes and the 16-byte reads free of bank conflicts, and the key order matches the k slots in
-    //    which the first product leaves the probabilities (lane half hh owns keys 4*hh + {0..3, 8..11} of a group).
-    const int ldC = tid % 16;
-    const int ldR = tid / 16;
-    const int q4 = lane / 16;
-    constexpr int kRowsPerPass = kThreads / 16;         // K rows covered by one pass of the work-group
-    constexpr int kKPasses = kBN / kRowsPerPass;        // 4 (256 threads) or 2 (512 threads)
-    constexpr int kVItems = (kBN / 2) * 16 / kThreads;  // (key pair, packet) items per thread: 2 or 1
-    u32x4 kReg[kKPasses], vReg[kVItems][2];
-    auto loadTile = [&](int jt) {
+    // ---- tile staging: 16-byte loads that land in LDS directly (no registers, no LDS write instructions) ----
+    // One such load of a wave fills 1 KB of consecutive LDS (lane l writes bytes 16 l .. 16 l + 15), i.e. 4 rows of
+    // a [64 keys][256 bytes] tile; which 16-byte packet of its row a lane fetches is free, and that is where the
+    // bank-conflict avoidance goes, since the rows cannot be padded:
+    //   K tile: slot s of row r holds packet s ^ (r & 15)      (16 lanes reading one packet of 16 rows hit 16 slots)
+    //   V tile: slot s of row r holds packet s ^ (4 * (r & 3)) (see the transposing reads below)
+    // Rows past the sequence are outside the tile's buffer descriptor and arrive as zeros; they are masked below.
+    constexpr int kTileBytes = kBN * kHD * static_cast<int>(sizeof(T));  // 16 KB
+    constexpr int kBufBytes = 2 * kTileBytes;                          // K tile, then V tile
+    constexpr int kChunks = kBN / 4 / NWV;                             // 1 KB pieces per wave and tile: 4 or 2
+    using LdsByte = __attribute__((address_space(3))) unsigned char;
+    LdsByte* const lds = (LdsByte*)dynSmem;
+    const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const int waveU = __builtin_amdgcn_readfirstlane(wave);
+    const int rowBytes = static_cast<int>(rowPitch) * static_cast<int>(sizeof(T));  // the launcher bounds 64 rows by 2^31 bytes
+    int kSrc[kChunks], vSrc[kChunks];
 #pragma unroll
-        for (int it = 0; it < kKPasses; ++it) {
-            int row = jt * kBN + ldR + it * kRowsPerPass;
-            row = row < L ? row : L - 1;  // keeps the load in bounds; such keys are masked below
-            kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
-        }
+    for (int it = 0; it < kChunks; ++it) {
+        const int r = (waveU * kChunks + it) * 4 + lane / 16;
+        kSrc[it] = r * rowBytes + (((lane % 16) ^ (r & 15)) * 16);
+        vSrc[it] = r * rowBytes + (((lane % 16) ^ (4 * (r & 3))) * 16);
+    }
+    // Requests tile jt into buffer jt & 1.  Unconditional: past the last tile it fetches the last tile again, into
+    // the buffer nobody reads any more.
+    auto requestTile = [&](int jt) {
+        const int jtL = jt < numKeyTiles ? jt : numKeyTiles - 1;
+        const int rowsLeft = L - jtL * kBN;
+        const int valid = rowsLeft < kBN ? rowsLeft : kBN;
+        const int bytes = static_cast<int>(((valid - 1) * rowPitch + kHD) * static_cast<int64_t>(sizeof(T)));
+        const uint64_t kAddr = reinterpret_cast<uint64_t>(kBase + jtL * kBN * rowPitch);
+        const uint64_t vAddr = reinterpret_cast<uint64_t>(vBase + jtL * kBN * rowPitch);
+        const u32x4 kBuf = {static_cast<uint32_t>(kAddr), static_cast<uint32_t>(kAddr >> 32) & 0xffffu, static_cast<uint32_t>(bytes), kRawBufferWord3};
+        const u32x4 vBuf = {static_cast<uint32_t>(vAddr), static_cast<uint32_t>(vAddr >> 32) & 0xffffu, static_cast<uint32_t>(bytes), kRawBufferWord3};
+        const uint32_t dst = ldsBase + (jt & 1) * kBufBytes + waveU * kChunks * 1024;
 #pragma unroll
-        for (int it = 0; it < kVItems; ++it) {
-            const int ci = wave * kVItems + it;  // 0..7: 16-key group ci / 2, half ci % 2
-#pragma unroll
-            for (int h2 = 0; h2 < 2; ++h2) {
-                int row = jt * kBN + 16 * (ci / 2) + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * (ci % 2) + h2;
-                row = row < L ? row : L - 1;
-                vReg[it][h2] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
-            }
-        }
-    };
-    auto stageTile = [&](int buf) {
-        T* sK = smem + buf * kStageElems;
-        uint32_t* sVt32 = reinterpret_cast<uint32_t*>(sK + kBN * kLD);
-#pragma unroll
-        for (int it = 0; it < kKPasses; ++it) *reinterpret_cast<u32x4*>(sK + (ldR + it * kRowsPerPass) * kLD + ldC * 8) = kReg[it];
-#pragma unroll
-        for (int it = 0; it < kVItems; ++it) {
-            const int ci = wave * kVItems + it;
-            const int posd = 8 * (ci / 2) + 4 * (ci % 2) + q4;  // dword position of this key pair inside a row
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t pair = __builtin_amdgcn_perm(vReg[it][1][e / 2], vReg[it][0][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
-                sVt32[(16 * e + ldC) * (kVP / 2) + posd] = pair;
-            }
+        for (int it = 0; it < kChunks; ++it) {
+            loadToLds16(kBuf, dst + it * 1024, kSrc[it]);
+            loadToLds16(vBuf, dst + kTileBytes + it * 1024, vSrc[it]);
         }
     };
-    // The same staging work cut into pieces of one or two instructions each, so that it can be dealt out between the
-    // matrix instructions of the second product: first the LDS writes of tile jt+1 (registers requested one iteration
-    // ago), then the global requests of tile jt+2 into the same registers.  Unconditional: rows are clamped and a
-    // surplus tile lands in a buffer nobody reads any more.
-    constexpr int kPiecesVW = 8 * kVItems, kPiecesKW = kKPasses, kPiecesKL = kKPasses, kPiecesVL = 2 * kVItems;
-    constexpr int kPieces = kPiecesVW + kPiecesKW + kPiecesKL + kPiecesVL;
-    auto stagePiece = [&](int idx, int jt) {
-        T* sKn = smem + ((jt + 1) & 1) * kStageElems;
-        if (idx < kPiecesVW) {
-            const int it = idx / 8, e = idx % 8;
-            const int ci = wave * kVItems + it;
-            const int posd = 8 * (ci / 2) + 4 * (ci % 2) + q4;
-            uint32_t* sVt32 = reinterpret_cast<uint32_t*>(sKn + kBN * kLD);
-            sVt32[(16 * e + ldC) * (kVP / 2) + posd] =
-                __builtin_amdgcn_perm(vReg[it][1][e / 2], vReg[it][0][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
-        } else if (idx < kPiecesVW + kPiecesKW) {
-            const int it = idx - kPiecesVW;
-            *reinterpret_cast<u32x4*>(sKn + (ldR + it * kRowsPerPass) * kLD + ldC * 8) = kReg[it];
-        } else if (idx < kPiecesVW + kPiecesKW + kPiecesKL) {
-            const int it = idx - kPiecesVW - kPiecesKW;
-            int row = (jt + 2) * kBN + ldR + it * kRowsPerPass;
-            row = row < L ? row : L - 1;
-            kReg[it] = *reinterpret_cast<const u32x4*>(kBase + row * rowPitch + ldC * 8);
-        } else if (idx < kPieces) {
-            const int k2 = idx - kPiecesVW - kPiecesKW - kPiecesKL;
-            const int it = k2 / 2, h2 = k2 % 2;
-            const int ci = wave * kVItems + it;
-            int row = (jt + 2) * kBN + 16 * (ci / 2) + 2 * (q4 & 1) + 8 * (q4 >> 1) + 4 * (ci % 2) + h2;
-            row = row < L ? row : L - 1;
-            vReg[it][h2] = *reinterpret_cast<const u32x4*>(vBase + row * rowPitch + ldC * 8);
-        }
-    };
-    loadTile(0);
-    stageTile(0);
-    loadTile(1);
+    requestTile(0);
+    // ---- operand addresses inside a buffer ----
+    // K (A operand of S^T): row 32 sb + n, packet 2 st + hh, one 16-byte read.
+    // V^T (A operand of O^T): a lane needs 8 keys of one dim, which in the row-major V tile are 8 rows apart by 256
+    // bytes.  The transposing read ds_read_b64_tr_b16 does the gather: inside a group of 16 lanes, lane (kk, q)
+    // (= lane % 16 / 4, lane % 4) supplies the address of 4 consecutive dims of key kk, and lane i receives element
+    // i % 4 of the 4 addresses given by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12: keys 0..3 of dim 4 (i / 4) + i % 4.
+    // Lane group g16 = lane / 16 covers dims 16 (g16 % 2) .. + 15 of a 32-dim block and keys 4 hh .. + 3 of an 8-key
+    // half; two reads (halves 0 and 1) give the 8 k slots of a lane in the order in which the first product leaves
+    // the probabilities (k slot (hh, j) of a 16-key group is key 8 (j / 4) + 4 hh + j % 4).  The 4 * (r & 3) swizzle
+    // spreads the 4 keys x 4 packets that 32 lanes touch at once over 16 different slots.
+    int kOff[kHD / 16], vOff[kHD / 32];
+    {
+        const int hx = hh ^ (n & 15);
+#pragma unroll
+        for (int st = 0; st < kHD / 16; ++st) kOff[st] = n * 256 + (((2 * st) ^ hx) * 16);
+        const int g16 = lane / 16, kk = (lane % 16) / 4, qq = lane % 4;
+        const int cLo = 2 * (g16 % 2) + qq / 2;
+#pragma unroll
+        for (int mb = 0; mb < kHD / 32; ++mb) vOff[mb] = kTileBytes + (4 * hh + kk) * 256 + ((4 * (mb ^ kk) + cLo) * 16) + (qq % 2) * 8;
+    }
+
+    // The query fragments must have arrived before the loop: a wait for them inside it would also wait for the tile
+    // requests, which the compiler does not count.
+#pragma unroll
+    for (int s = 0; s < kHD / 16; ++s) asm volatile("" : "+v"(qf[s]));
 
     for (int jt = 0; jt < numKeyTiles; ++jt) {
-        // One barrier per tile: tile jt is staged and every wave has left tile jt-1, whose buffer now takes tile
-        // jt+1 (requested one iteration ago, so its latency is covered); the request for tile jt+2 follows.
+        // One barrier per tile: tile jt has landed (every wave waits for its own requests before the barrier) and
+        // every wave has left tile jt-1, whose buffer the request for tile jt+1 now fills while this tile is used.
+        waitLdsLoads();
         __syncthreads();
-        const T* sK = smem + (jt & 1) * kStageElems;
-        const T* sVt = sK + kBN * kLD;
+        requestTile(jt + 1);
+        const LdsByte* sBuf = lds + (jt & 1) * kBufBytes;
 
         const int key0 = jt * kBN;
-        if (causal && key0 > waveRowHi) {
-            // entirely above the diagonal for this wave: only the staging duty remains
-#pragma unroll
-            for (int idx = 0; idx < kPieces; ++idx) stagePiece(idx, jt);
-            continue;
-        }  // entirely above the diagonal for this wave (barriers are at the loop top)
+        if (causal && key0 > waveRowHi) continue;  // entirely above the diagonal for this wave (barriers are at the loop top)
 
         // ---- S^T = K . Q^T for the two 32-key blocks ----
         // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
@@ -331,7 +318,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         FragBits<Frag> kf[kKDepth][2];
         auto loadK = [&](int st, int b) {
 #pragma unroll
-            for (int sb = 0; sb < 2; ++sb) kf[b][sb].raw = *reinterpret_cast<const u32x4*>(sK + (sb * 32 + n) * kLD + st * 16 + hh * 8);
+            for (int sb = 0; sb < 2; ++sb) kf[b][sb].raw = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(sBuf + kOff[st] + sb * 32 * 256);
         };
 #pragma unroll
         for (int st = 0; st < kKDepth - 1; ++st) loadK(st, st);
@@ -347,7 +334,15 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         FragBits<Frag> vf[2][kHD / 32];
         auto loadV = [&](int g, int b) {
 #pragma unroll
-            for (int mb = 0; mb < kHD / 32; ++mb) vf[b][mb].raw = *reinterpret_cast<const u32x4*>(sVt + (32 * mb + n) * kVP + 16 * g + 8 * hh);
+            for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    using Quad = __attribute__((address_space(3))) s16x4;
+                    const s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((Quad*)(sBuf + vOff[mb] + (16 * g + 8 * h2) * 256));
+                    vf[b][mb].raw[2 * h2] = __builtin_bit_cast(u32x2, t)[0];
+                    vf[b][mb].raw[2 * h2 + 1] = __builtin_bit_cast(u32x2, t)[1];
+                }
+            }
         };
         loadV(0, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -403,21 +398,14 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         }
         lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
         // ---- O^T += V^T . P^T : k slot (hh, j) of group g = 2*sb + u is key 16*g + 8*(j/4) + 4*hh + j%4 ----
-        // accumulator row n' of o[mb] stands for LDS row 32*mb + n', i.e. dim 8 * (row % 16) + row / 16
+        // accumulator row n' of o[mb] stands for dim 32*mb + n'
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (g + 1 < 4) loadV(g + 1, (g + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mb = 0; mb < kHD / 32; ++mb) {
-                o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
-                // staging pieces ride in the shadow of the matrix instruction just issued (the buffer of tile jt-1
-                // is free since this iteration's barrier)
-                constexpr int kPerSlot = (kPieces + 15) / 16;
-#pragma unroll
-                for (int k2 = 0; k2 < kPerSlot; ++k2) stagePiece((g * 4 + mb) * kPerSlot + k2, jt);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
@@ -429,20 +417,19 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         if (a.lse != nullptr && hh == 0 && qRow < L && qRow < a.lseStride)
             a.lse[(static_cast<int64_t>(planned.x) * a.H + head) * a.lseStride + qRow] = 0.6931471805599453f * (mRun * scaleLog2 + __builtin_amdgcn_logf(lTot));
     }
-    __syncthreads();  // the K/V tiles are dead; reuse the storage as a [BM][kLD] output tile
+    waitLdsLoads();
+    __syncthreads();  // the K/V tiles are dead (and the surplus request has landed); reuse the storage as a [BM][kLD] output tile
     T* sO = smem;
     static_assert(kHD == 128, "scaleLog2 is written out for head size 128");
-    static_assert(BM * kLD <= 2 * kStageElems, "the output tile must fit the staging storage");
 #pragma unroll
     for (int mb = 0; mb < kHD / 32; ++mb) {
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            // registers r and r + 8 of o[mb] are LDS rows 32*mb + 8*(r/4) + 4*hh + r%4 (+16): dims d and d + 1
-            const int d = 64 * ((r >> 2) & 1) + 32 * hh + 8 * (r & 3) + 2 * mb;
-            T pk[2];
-            pk[0] = static_cast<T>(o[mb][r] * inv);
-            pk[1] = static_cast<T>(o[mb][r + 8] * inv);
-            *reinterpret_cast<uint32_t*>(sO + (wave * 32 + n) * kLD + d) = *reinterpret_cast<const uint32_t*>(pk);
+        for (int rq = 0; rq < 4; ++rq) {
+            // registers 4 rq .. 4 rq + 3 of o[mb] are dims 32 mb + 8 rq + 4 hh .. + 3
+            T pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = static_cast<T>(o[mb][4 * rq + e] * inv);
+            *reinterpret_cast<u32x2*>(sO + (wave * 32 + n) * kLD + 32 * mb + 8 * rq + 4 * hh) = *reinterpret_cast<const u32x2*>(pk);
         }
     }
     // each wave only reads back the 32 rows it wrote: no work-group barrier needed, LDS ops of a wave are ordered
@@ -538,7 +525,8 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles, BM);
     ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
-    constexpr int ldsBytes = 2 * kStageElems * static_cast<int>(sizeof(T));
+    constexpr int kStaging = 2 * 2 * kBN * kHD, kOutTile = BM * kLD;  // elements: two (K, V) buffers; the output tile that reuses them
+    constexpr int ldsBytes = (kStaging > kOutTile ? kStaging : kOutTile) * static_cast<int>(sizeof(T));
     static hipError_t granted =
         hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV, GEN>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
     ROCM_HIP(granted);
@@ -570,7 +558,9 @@ diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, con
         ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
     // the planning kernel keeps two ints per sequence and one per query tile in LDS
     const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
-    const bool fast = D == kHD && aligned && planFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    // the tile requests address a 64-row tile with 32-bit byte offsets
+    const bool tileFits = static_cast<int64_t>(a.H) * kHD * 8 * kBN < INT32_MAX;
+    const bool fast = D == kHD && aligned && planFits && tileFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
     // 256-row query tiles (8 waves share each K/V tile) once the sequences are long enough to fill them
     const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
     switch (vQ.dtype) {
