@@ -321,7 +321,26 @@ def main():
         hsrc, hperm, hcache = Tensor(src), Tensor(perm), Tensor(w3["k_cache"])
         ms = timed(lambda i: check(impl.diopiDestIndexCopyKV(ctx.handle, hcache.handle, hsrc.handle, hperm.handle), "diopiDestIndexCopyKV"))
         record("diopiDestIndexCopyKV", f"sweep: {Tn} tokens x 8 KiB", ms, W.destindex_bytes(Tn, 32, 128, 2), "hbm", "f16")
-        del w3, src, perm, hsrc, hperm, hcache
+        # the same decode step through the paged-attention interface: the cache as 1024 blocks of 128 rows, each sequence
+        # on 16 blocks drawn from a random permutation, its cfg3 length; both decode kernels plus the table expansion
+        B3, H3, D3 = w3["B"], w3["H"], w3["D"]
+        lens3 = [int(x) for x in w3["b_seq_len"].cpu()]
+        table = torch.randperm(1024, device=dev).int().view(B3, 16)
+        q2, k2, v2 = w3["q"].view(B3, H3 * D3), w3["k_cache"].view(-1, H3 * D3), w3["v_cache"].view(-1, H3 * D3)
+        o2 = torch.zeros_like(q2)
+        hp = {k: Tensor(v) for k, v in dict(q=q2, k=k2, v=v2, o=o2, t=table).items()}
+        sz = rt.Sizes(lens3)
+
+        def paged(i):
+            check(impl.diopiPagedAttention(ctx.handle, hp["o"].handle, hp["q"].handle, hp["k"].handle, hp["v"].handle, None, sz.c, H3, H3, D3,
+                                           hp["t"].handle, 128), "diopiPagedAttention")
+            ctx.clear_tensors()
+
+        ms_pg = timed(paged)
+        e_pg = record("diopiPagedAttention (blocks of 128 rows)", f"cfg3 lengths fp16 B={B3}", ms_pg, head["b_att"] + head["b_red"], "hbm", "f16", None,
+                      note="widening beyond the seven hot-path operators; block table -> row table, then the two decode kernels")
+        e_pg["tokens_per_s"] = round(B3 / (ms_pg * 1e-3), 1)
+        del w3, src, perm, hsrc, hperm, hcache, hp, q2, k2, v2, o2, table
         torch.cuda.empty_cache()
 
     if not only or "cfg5" in only:

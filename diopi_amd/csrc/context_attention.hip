@@ -847,3 +847,70 @@ extern "C" diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t ctx, 
     return attentionVarLen(ctx, "diopiMultiHeadAttentionVarLen", out, softmax_lse, q, k, v, cum_seq_q, cum_seq_k, max_q, scale, is_causal);
     ROCM_ENTRY_END
 }
+
+// Causal prefill on a padded batch with flattened heads (proto/include/diopi/functions_ext.h:684-686; Python statement
+// customized_test.py:751-780): query and out are [batch * max_input_len, num_heads * dim], key and value
+// [batch * max_input_len, num_kv_heads * dim]; sequence i owns rows [i * max_input_len, (i + 1) * max_input_len) and
+// every row attends to the rows of its sequence up to its own.  Like the statement, this takes only the batch size
+// from actual_seq_lengths and computes every row (under the causal mask the rows inside a shorter actual length do
+// not depend on the padding behind them), and it does not read atten_mask: the statement builds the lower-triangular
+// mask itself.
+extern "C" diopiError_t diopiPromptFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t query,
+                                                  diopiConstTensorHandle_t key, diopiConstTensorHandle_t value, diopiConstTensorHandle_t atten_mask,
+                                                  diopiSize_t actual_seq_lengths, int64_t max_input_len, int64_t num_heads, int64_t num_kv_heads, int64_t dim) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)atten_mask;
+    TensorView vOut, vQ, vK, vV;
+    ROCM_CALL(unwrap(out, "out", &vOut));
+    ROCM_CALL(unwrap(query, "query", &vQ));
+    ROCM_CALL(unwrap(key, "key", &vK));
+    ROCM_CALL(unwrap(value, "value", &vV));
+    ROCM_CALL(requireDeviceContiguous(vOut, "out"));
+    ROCM_CALL(requireDeviceContiguous(vQ, "query"));
+    ROCM_CALL(requireDeviceContiguous(vK, "key"));
+    ROCM_CALL(requireDeviceContiguous(vV, "value"));
+    ROCM_CHECK(num_heads > 0 && num_kv_heads > 0 && dim > 0 && num_heads % num_kv_heads == 0 && num_heads <= INT32_MAX / 1024 && dim <= 65535,
+               "num_heads %lld must be a positive multiple of num_kv_heads %lld, dim %lld positive", static_cast<long long>(num_heads),
+               static_cast<long long>(num_kv_heads), static_cast<long long>(dim));
+    ROCM_CHECK(actual_seq_lengths.len >= 0 && actual_seq_lengths.len <= 65535 && max_input_len >= 0 && max_input_len <= INT32_MAX,
+               "batch size %lld or max_input_len %lld out of range", static_cast<long long>(actual_seq_lengths.len), static_cast<long long>(max_input_len));
+    const int64_t batch = actual_seq_lengths.len;
+    const int64_t rows = batch * max_input_len;
+    ROCM_CHECK(vQ.ndim == 2 && vQ.shape[0] == rows && vQ.shape[1] == num_heads * dim, "query must be [batch * max_input_len, num_heads * dim] = [%lld, %lld]",
+               static_cast<long long>(rows), static_cast<long long>(num_heads * dim));
+    ROCM_CHECK(vOut.sameShape(vQ), "out must have the shape of query");
+    ROCM_CHECK(vK.ndim == 2 && vK.shape[0] == rows && vK.shape[1] == num_kv_heads * dim && vV.sameShape(vK),
+               "key and value must be [batch * max_input_len, num_kv_heads * dim] = [%lld, %lld]", static_cast<long long>(rows),
+               static_cast<long long>(num_kv_heads * dim));
+    ROCM_CHECK(isFloatDtype(vQ.dtype) && vK.dtype == vQ.dtype && vV.dtype == vQ.dtype && vOut.dtype == vQ.dtype,
+               "query, key, value and out must share one floating dtype (query is %s)", dtypeName(vQ.dtype));
+    if (rows == 0) return diopiSuccess;
+
+    CtxArgs a;
+    a.bStartLoc = nullptr;
+    a.bSeqLen = nullptr;
+    a.start64 = false;
+    a.len64 = false;
+    a.batch = static_cast<int>(batch);
+    a.H = static_cast<int>(num_heads);
+    a.rows = rows;
+    a.tilesBound = 0;
+    a.totalItems = 0;
+    a.cumulative = false;
+    a.uniformLen = static_cast<int>(max_input_len);
+    a.causal = true;
+    a.G = static_cast<int>(num_heads / num_kv_heads);
+    const int D = static_cast<int>(dim);
+    const double scale = 1.0 / std::sqrt(static_cast<double>(D));
+    a.scaleLog2 = static_cast<float>(scale * 1.4426950408889634);
+    a.lse = nullptr;
+    a.lseStride = 0;
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    const diopiError_t err = dispatchAttention<true>(ctx, stream, vOut, vQ, vK, vV, a, D, scale);
+    if (err != diopiDtypeNotSupported) return err;
+    setLastError("diopiPromptFlashAttention: dtype %s is not supported", dtypeName(vQ.dtype));
+    return diopiDtypeNotSupported;
+    ROCM_ENTRY_END
+}

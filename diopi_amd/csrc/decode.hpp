@@ -27,6 +27,14 @@ struct DecodeArgs {
 diopiError_t prepareDecode(const TensorView& logits, const TensorView& qOrOut, const TensorView& cache, const TensorView& bLoc, const TensorView& bStartLoc,
                            const TensorView& bSeqLen, int maxInputLen, DecodeArgs* args, bool* empty);
 
+// The two decode operators on tensor views (what the C entry points call after unwrapping their handles, and what
+// diopiPagedAttention calls on views of its own scratch tensors).  `out`/`logits` is [H, cols], q/out is [B, H, D],
+// the cache is [slots, Hkv, D].
+diopiError_t tokenAttention(diopiContextHandle_t ctx, const TensorView& out, const TensorView& q, const TensorView& k, const TensorView& bLoc,
+                            const TensorView& bStartLoc, const TensorView& bSeqLen, int maxInputLen);
+diopiError_t tokenSoftmaxReduceV(diopiContextHandle_t ctx, const TensorView& out, const TensorView& logits, const TensorView& v, const TensorView& bLoc,
+                                 const TensorView& bStartLoc, const TensorView& bSeqLen, int maxInputLen);
+
 }  // namespace rocm
 
 #endif  // DIOPI_ROCM_CSRC_DECODE_HPP_

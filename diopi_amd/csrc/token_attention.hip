@@ -378,18 +378,10 @@ diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const v
 }  // namespace
 }  // namespace rocm
 
-extern "C" diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t token_attention_out, diopiConstTensorHandle_t q,
-                                                     diopiConstTensorHandle_t k, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
-                                                     diopiConstTensorHandle_t b_seq_len, int max_input_len) {
-    ROCM_ENTRY_BEGIN
-    using namespace rocm;
-    TensorView vOut, vQ, vK, vLoc, vStart, vLen;
-    ROCM_CALL(unwrap(token_attention_out, "token_attention_out", &vOut));
-    ROCM_CALL(unwrap(q, "q", &vQ));
-    ROCM_CALL(unwrap(k, "k", &vK));
-    ROCM_CALL(unwrap(b_loc, "b_loc", &vLoc));
-    ROCM_CALL(unwrap(b_start_loc, "b_start_loc", &vStart));
-    ROCM_CALL(unwrap(b_seq_len, "b_seq_len", &vLen));
+namespace rocm {
+
+diopiError_t tokenAttention(diopiContextHandle_t ctx, const TensorView& vOut, const TensorView& vQ, const TensorView& vK, const TensorView& vLoc,
+                            const TensorView& vStart, const TensorView& vLen, int max_input_len) {
     DecodeArgs a;
     bool empty = false;
     ROCM_CALL(prepareDecode(vOut, vQ, vK, vLoc, vStart, vLen, max_input_len, &a, &empty));
@@ -416,5 +408,22 @@ extern "C" diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, d
     }
     setLastError("diopiTokenAttentionInference: dtype %s is not supported", dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
+}
+
+}  // namespace rocm
+
+extern "C" diopiError_t diopiTokenAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t token_attention_out, diopiConstTensorHandle_t q,
+                                                     diopiConstTensorHandle_t k, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
+                                                     diopiConstTensorHandle_t b_seq_len, int max_input_len) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    TensorView vOut, vQ, vK, vLoc, vStart, vLen;
+    ROCM_CALL(unwrap(token_attention_out, "token_attention_out", &vOut));
+    ROCM_CALL(unwrap(q, "q", &vQ));
+    ROCM_CALL(unwrap(k, "k", &vK));
+    ROCM_CALL(unwrap(b_loc, "b_loc", &vLoc));
+    ROCM_CALL(unwrap(b_start_loc, "b_start_loc", &vStart));
+    ROCM_CALL(unwrap(b_seq_len, "b_seq_len", &vLen));
+    return tokenAttention(ctx, vOut, vQ, vK, vLoc, vStart, vLen, max_input_len);
     ROCM_ENTRY_END
 }

@@ -507,19 +507,10 @@ diopiError_t launchGeneric(hipStream_t stream, void* out, const void* logits, co
 }  // namespace
 }  // namespace rocm
 
-extern "C" diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t logics,
-                                                          diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
-                                                          diopiConstTensorHandle_t b_seq_len, int max_input_len, int other_kv_index) {
-    ROCM_ENTRY_BEGIN
-    using namespace rocm;
-    (void)other_kv_index;  // unused by the reference as well (functions_lightllm.cpp:82-107)
-    TensorView vOut, vLogits, vV, vLoc, vStart, vLen;
-    ROCM_CALL(unwrap(out, "out", &vOut));
-    ROCM_CALL(unwrap(logics, "logics", &vLogits));
-    ROCM_CALL(unwrap(v, "v", &vV));
-    ROCM_CALL(unwrap(b_loc, "b_loc", &vLoc));
-    ROCM_CALL(unwrap(b_start_loc, "b_start_loc", &vStart));
-    ROCM_CALL(unwrap(b_seq_len, "b_seq_len", &vLen));
+namespace rocm {
+
+diopiError_t tokenSoftmaxReduceV(diopiContextHandle_t ctx, const TensorView& vOut, const TensorView& vLogits, const TensorView& vV, const TensorView& vLoc,
+                                 const TensorView& vStart, const TensorView& vLen, int max_input_len) {
     DecodeArgs a;
     bool empty = false;
     ROCM_CALL(prepareDecode(vLogits, vOut, vV, vLoc, vStart, vLen, max_input_len, &a, &empty));
@@ -544,5 +535,23 @@ extern "C" diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t c
     }
     setLastError("diopiTokenSoftmaxReduceVInference: dtype %s is not supported", dtypeName(vOut.dtype));
     return diopiDtypeNotSupported;
+}
+
+}  // namespace rocm
+
+extern "C" diopiError_t diopiTokenSoftmaxReduceVInference(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t logics,
+                                                          diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_loc, diopiConstTensorHandle_t b_start_loc,
+                                                          diopiConstTensorHandle_t b_seq_len, int max_input_len, int other_kv_index) {
+    ROCM_ENTRY_BEGIN
+    using namespace rocm;
+    (void)other_kv_index;  // unused by the reference as well (functions_lightllm.cpp:82-107)
+    TensorView vOut, vLogits, vV, vLoc, vStart, vLen;
+    ROCM_CALL(unwrap(out, "out", &vOut));
+    ROCM_CALL(unwrap(logics, "logics", &vLogits));
+    ROCM_CALL(unwrap(v, "v", &vV));
+    ROCM_CALL(unwrap(b_loc, "b_loc", &vLoc));
+    ROCM_CALL(unwrap(b_start_loc, "b_start_loc", &vStart));
+    ROCM_CALL(unwrap(b_seq_len, "b_seq_len", &vLen));
+    return tokenSoftmaxReduceV(ctx, vOut, vLogits, vV, vLoc, vStart, vLen, max_input_len);
     ROCM_ENTRY_END
 }

@@ -248,3 +248,33 @@ def multihead_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
     check_returncode(ret, "diopiMultiHeadAttentionVarLen")
     GLOBAL_STATE["multihead_attention_varlen_softmax_lse"] = lse
     return out
+
+
+def prompt_flash_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attenMask: Optional[torch.Tensor], actualSeqLengths: Sequence[int],
+                           maxInputLen: int, numHeads: int, numKeyValueHeads: int, dim: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py:7951-7981 of the reference."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(query)
+    sizes = Sizes(actualSeqLengths)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, query, key, value, attenMask)
+        ret = rt.libs().impl.diopiPromptFlashAttention(ctx.handle, h[0], h[1], h[2], h[3], h[4], sizes.c, int(maxInputLen), int(numHeads),
+                                                       int(numKeyValueHeads), int(dim))
+    check_returncode(ret, "diopiPromptFlashAttention")
+    return out
+
+
+def paged_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attenMask: Optional[torch.Tensor], actualSeqLengths: Sequence[int],
+                    numHeads: int, numKeyValueHeads: int, dim: int, blockTable: torch.Tensor, blockSize: int,
+                    ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """diopi_functions.py:7984-8016 of the reference."""
+    ctx = _ctx(ctx)
+    out = torch.empty_like(query)
+    sizes = Sizes(actualSeqLengths)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, query, key, value, attenMask, blockTable)
+        ret = rt.libs().impl.diopiPagedAttention(ctx.handle, h[0], h[1], h[2], h[3], h[4], sizes.c, int(numHeads), int(numKeyValueHeads), int(dim), h[5],
+                                                 int(blockSize))
+    ctx.clear_tensors()
+    check_returncode(ret, "diopiPagedAttention")
+    return out

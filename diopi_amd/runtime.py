@@ -150,6 +150,8 @@ class _Libs:
         i64, dbl = ctypes.c_int64, ctypes.c_double
         impl.diopiMultiHeadAttention.argtypes = [vp, vp, vp, vp, dbl, ctypes.c_bool, ctypes.c_bool, dbl, vp, vp, vp, vp]
         impl.diopiMultiHeadAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ctypes.c_bool, ctypes.c_bool, dbl, vp, vp, vp, vp]
+        impl.diopiPagedAttention.argtypes = [vp, vp, vp, vp, vp, vp, _SizeStruct, i64, i64, i64, vp, i64]
+        impl.diopiPromptFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, _SizeStruct, i64, i64, i64, i64]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
@@ -170,6 +172,8 @@ OPERATOR_SYMBOLS = (
     "diopiFlashAttention",
     "diopiMultiHeadAttention",
     "diopiMultiHeadAttentionVarLen",
+    "diopiPagedAttention",
+    "diopiPromptFlashAttention",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

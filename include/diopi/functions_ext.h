@@ -181,6 +181,30 @@ DIOPI_API diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t ctx, d
                                                      double dropout_p, bool is_causal, bool return_debug_mask, double scale, diopiTensorHandle_t out,
                                                      diopiTensorHandle_t softmax_lse, diopiGeneratorHandle_t gen, diopiTensorHandle_t debug_attn_mask);
 
+/*
+ * One decode step of attention over a KV cache cut into blocks.
+ * reference: functions_ext.h:602-618 (Python statement customized_test.py:782-821; case diopi_configs.py:9425-9468).
+ * q, out [batch, num_heads * dim]; k, v [rows, num_kv_heads * dim]; num_heads a multiple of num_kv_heads; block_table
+ * int32 or int64 [batch, blocks]; actual_seq_lengths a host list of batch token counts.  Token t of sequence i is row
+ * block_table[i, t / block_size] * block_size + t % block_size of k and v; out[i, h] = softmax(q[i, h] . K^T / sqrt(dim)) V
+ * over that sequence's tokens.  attenMask is not read (the statement does not read it either).  Asynchronous on the
+ * context's stream; the host list is consumed before the call returns.
+ */
+DIOPI_API diopiError_t diopiPagedAttention(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                                           diopiConstTensorHandle_t v, diopiConstTensorHandle_t attenMask, diopiSize_t actual_seq_lengths, int64_t num_heads,
+                                           int64_t num_kv_heads, int64_t dim, diopiConstTensorHandle_t block_table, int64_t block_size);
+
+/*
+ * Causal prefill attention on a padded batch with flattened heads.
+ * reference: functions_ext.h:684-686 (Python statement customized_test.py:751-780; case diopi_configs.py:9383-9423).
+ * query, out [batch * max_input_len, num_heads * dim]; key, value [batch * max_input_len, num_kv_heads * dim]; batch is
+ * the length of the host list actual_seq_lengths.  Row r of sequence i attends to rows 0..r of that sequence, scale
+ * 1/sqrt(dim).  As in the statement every row is computed and atten_mask is not read.
+ */
+DIOPI_API diopiError_t diopiPromptFlashAttention(diopiContextHandle_t ctx, diopiTensorHandle_t out, diopiConstTensorHandle_t query,
+                                                 diopiConstTensorHandle_t key, diopiConstTensorHandle_t value, diopiConstTensorHandle_t atten_mask,
+                                                 diopiSize_t actual_seq_lengths, int64_t max_input_len, int64_t num_heads, int64_t num_kv_heads, int64_t dim);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -1,5 +1,5 @@
-"""CPU oracle for the LLaMA-inference operators (the seven of the hot path,
-diopiRotaryEmbeddingV2 and diopiApplyPenalty/V2).  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the LLaMA-inference operators (the seven of the hot path, diopiRotaryEmbeddingV2,
+diopiApplyPenalty/V2 and the flash / prompt / paged attention forms).  TEST INFRASTRUCTURE ONLY.
 
 This module restates, on the CPU with plain ATen (torch) and numpy calls, what the reference
 computes for each operator.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
@@ -25,6 +25,9 @@ context_attention            functions_lightllm.cpp:109-147; customized_test.py:
 flash_attention              customized_test.py:462-485 (declaration functions_ext.h:209-212)
 flash_attention_varlen       customized_test.py:525-588 with multi_head_attention_inside, 36-57 (the torch
                              implementation calls the flash-attn library; declaration functions_ext.h:355-359)
+prompt_flash_attention       customized_test.py:751-780 (no torch body; declaration functions_ext.h:684-686)
+paged_attention              customized_test.py:782-821 (no torch body; declaration functions_ext.h:616-618),
+                             extended from its single in-order sequence to a block table per sequence
 ===========================  =====================================================================
 
 Two arithmetic modes:
@@ -67,6 +70,12 @@ How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"
   flash_attention_varlen  causal multi-head case = context_attention on the same tokens, identical keys ->
                        mean of the visible values and lse = scale*q.k + ln(count), explicit Python loops for
                        full attention, grouped heads, a custom scale and the log-sum-exp
+  prompt_flash_attention  agreement with context_attention on the same rows cut into equal sequences (two
+                       restatements written from different reference functions), first row of every sequence returns
+                       its v row, explicit Python loops with fewer key/value heads
+  paged_attention      the reference's case shape (diopi_configs.py:9425-9468: 5 tokens, blocks [0, 1]) against the
+                       statement's own reading (rows 0..4), shuffled block tables against explicit Python loops in
+                       float64, agreement with token_attention + token_softmax_reducev on the expanded row table
   context_attention    first token of every sequence returns its v row bit for bit, constant V,
                        the reference's ragged fixtures (diopi_configs.py:9349-9377) incl. untouched
                        rows, float64 brute force, and the last row cross-checked against
@@ -351,3 +360,61 @@ def flash_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, alibi_slo
             scores = scores + torch.triu(torch.full((seqlen, seqlen), float("-inf")), 1).to(dtype=scores.dtype)
         out = torch.einsum("bhts,bshd->bthd", torch.softmax(scores, dim=-1, dtype=v.dtype), v)
     return (out, lse) if return_lse else out
+
+
+def prompt_flash_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attenMask, actualSeqLengths: Sequence[int], maxInputLen: int,
+                           numHeads: int, numKeyValueHeads: int, dim: int, exact: bool = False) -> torch.Tensor:
+    """customized_test.py:751-780: every sequence is maxInputLen rows of the flattened [bs * maxInputLen, heads * dim]
+    tensors; lower-triangular mask built here (attenMask is not read), scores in the tensor dtype, fp32 softmax rounded
+    back, product with the values.  The statement's matmul broadcasts the key/value heads, which only works for
+    numKeyValueHeads in (numHeads, 1); other divisors repeat each key/value head numHeads / numKeyValueHeads times (the
+    grouping rule of customized_test.py:466-472), which agrees with the broadcast in both of those cases."""
+    bs = len(actualSeqLengths)
+    g = numHeads // numKeyValueHeads
+    xq = query.view(bs, maxInputLen, numHeads, dim).transpose(1, 2)
+    keys = key.view(bs, maxInputLen, numKeyValueHeads, dim).repeat_interleave(g, dim=2).transpose(1, 2)
+    values = value.view(bs, maxInputLen, numKeyValueHeads, dim).repeat_interleave(g, dim=2).transpose(1, 2)
+    if exact:
+        scores = torch.matmul(xq.double(), keys.double().transpose(2, 3)) / math.sqrt(dim)
+        masked = torch.triu(torch.ones(maxInputLen, maxInputLen, dtype=torch.bool), diagonal=1)
+        scores = scores.masked_fill(masked, float("-inf")).softmax(-1)
+        out = torch.matmul(scores, values.double()).transpose(1, 2).to(query.dtype)
+        return out.reshape(bs * maxInputLen, numHeads * dim)
+    mask = torch.tril(torch.ones(maxInputLen, maxInputLen), diagonal=0).unsqueeze(0).unsqueeze(0)
+    mask = mask.masked_fill(mask == 0.0, -100000000.0)
+    scores = torch.matmul(xq, keys.transpose(2, 3)) / math.sqrt(dim)
+    scores = torch.softmax(scores.float() + mask, dim=-1).type_as(xq)
+    out = torch.matmul(scores, values).transpose(1, 2).contiguous()
+    return out.reshape(bs * maxInputLen, numHeads * dim)
+
+
+def paged_rows(blockTable: torch.Tensor, i: int, L: int, blockSize: int) -> torch.Tensor:
+    """Rows of key/value that hold tokens 0..L-1 of sequence i: block_table[i, t // block_size] * block_size + t % block_size."""
+    t = torch.arange(L, dtype=torch.int64)
+    return blockTable[i].long()[t // blockSize] * blockSize + t % blockSize
+
+
+def paged_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attenMask, actualSeqLengths: Sequence[int], numHeads: int,
+                    numKeyValueHeads: int, dim: int, blockTable: torch.Tensor, blockSize: int, exact: bool = False) -> torch.Tensor:
+    """customized_test.py:782-821, per sequence: logits = q . K^T / sqrt(dim) in the tensor dtype, softmax in that dtype,
+    product with V.  The statement handles one sequence whose token t is row t of key/value; here sequence i's token t is
+    the row its block table names (paged_rows), which is row t for the statement's case (blocks 0, 1, ... in order).
+    attenMask is not read.  Sequences without tokens give zeros."""
+    batch = len(actualSeqLengths)
+    g = numHeads // numKeyValueHeads
+    cdt = torch.float64 if exact else query.dtype
+    xq = query.view(batch, 1, numHeads, dim).transpose(1, 2).to(cdt)  # [B, H, 1, D]
+    k = key.view(-1, numKeyValueHeads, dim)
+    v = value.view(-1, numKeyValueHeads, dim)
+    out = torch.zeros(batch, numHeads, dim, dtype=cdt)
+    for i in range(batch):
+        L = int(actualSeqLengths[i])
+        if L == 0:
+            continue
+        rows = paged_rows(blockTable, i, L, blockSize)
+        kk = k[rows].to(cdt).repeat_interleave(g, dim=1).view(1, L, numHeads, dim).transpose(1, 2)
+        logics = (torch.matmul(xq[i], kk.transpose(2, 3)) / math.sqrt(dim)).reshape(numHeads, L)
+        P = logics.softmax(-1).reshape(1, numHeads, 1, L)
+        V = v[rows].to(cdt).repeat_interleave(g, dim=1).view(1, L, numHeads, dim).transpose(1, 2)
+        out[i] = torch.matmul(P, V).view(numHeads, dim)
+    return out.to(query.dtype).view(-1, numHeads * dim)

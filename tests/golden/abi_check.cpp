@@ -44,6 +44,10 @@ diopiError_t diopiMultiHeadAttention(diopiContextHandle_t, diopiTensorHandle_t, 
 diopiError_t diopiMultiHeadAttentionVarLen(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t,
                                            diopiConstTensorHandle_t, int64_t, int64_t, double, bool, bool, double, diopiTensorHandle_t, diopiTensorHandle_t,
                                            diopiGeneratorHandle_t, diopiTensorHandle_t);
+diopiError_t diopiPagedAttention(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
+                                 diopiConstTensorHandle_t, diopiSize_t, int64_t, int64_t, int64_t, diopiConstTensorHandle_t, int64_t);
+diopiError_t diopiPromptFlashAttention(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t, diopiConstTensorHandle_t,
+                                       diopiConstTensorHandle_t, diopiSize_t, int64_t, int64_t, int64_t, int64_t);
 // the callbacks the library imports
 diopiError_t diopiGetTensorShape(diopiConstTensorHandle_t, diopiSize_t*);
 diopiError_t diopiGetStream(diopiContextHandle_t, diopiStreamHandle_t*);

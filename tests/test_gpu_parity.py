@@ -760,6 +760,71 @@ def test_multihead_attention_older_names():
         F.multihead_attention_varlen(qp, kp, vp, cu, 163, 0, True, True, None)
 
 
+# ----------------------------------------------------------------------------- prompt flash attention and paged attention
+def test_prompt_flash_attention_reference_case_and_long_prompts():
+    # the reference's case (diopi_configs.py:9383-9423): 2 sequences of 2 rows, 32 heads of 128, fp16, its boolean mask
+    g = gen(960)
+    q, k, v = ((torch.randn(4, 4096, generator=g) * 0.5).half().to(DEV) for _ in range(3))
+    mask = torch.tensor([[[False, True], [False, False]]] * 2, device=DEV)
+    out = F.prompt_flash_attention(q, k, v, mask, [2, 2], 2, 32, 32, 128)
+    assert out.shape == (4, 4096)
+    ref = O.prompt_flash_attention(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), [2, 2], 2, 32, 32, 128)
+    assert_close(out, ref, **TOL[torch.float16], what="prompt_flash_attention, reference case", mismatch_ratio=1e-3)
+    assert torch.equal(out[0].cpu(), v[0].cpu()) and torch.equal(out[2].cpu(), v[2].cpu())  # a first row is its own value row
+    # prompts long enough for the matrix-core kernel, fewer key/value heads, bf16 and fp32
+    for dtype, bs, L, H, Hkv, D in ((torch.float16, 3, 300, 8, 2, 128), (torch.bfloat16, 2, 257, 4, 4, 128), (torch.float32, 2, 40, 4, 2, 64)):
+        q = (torch.randn(bs * L, H * D, generator=g) * 0.5).to(dtype).to(DEV)
+        k = (torch.randn(bs * L, Hkv * D, generator=g) * 0.5).to(dtype).to(DEV)
+        v = (torch.randn(bs * L, Hkv * D, generator=g) * 0.5).to(dtype).to(DEV)
+        out = F.prompt_flash_attention(q, k, v, None, [L, L - 1, 1][:bs], L, H, Hkv, D)
+        exact = O.prompt_flash_attention(q.cpu(), k.cpu(), v.cpu(), None, [L] * bs, L, H, Hkv, D, exact=True)
+        assert_close(out, exact, **TOL[dtype], what=f"prompt_flash_attention {dtype}")
+    with pytest.raises(rt.DiopiException):
+        F.prompt_flash_attention(q, k, v, None, [40, 40, 40], 40, 4, 2, 64)  # rows do not match batch * max_input_len
+    with pytest.raises(rt.DiopiException):
+        F.prompt_flash_attention(q, k, v, None, [40, 40], 40, 4, 3, 64)  # heads not a multiple of key/value heads
+    assert F.prompt_flash_attention(q[:0], k[:0], v[:0], None, [], 40, 4, 2, 64).numel() == 0
+
+
+def test_paged_attention_reference_case_and_block_tables():
+    # the reference's case (diopi_configs.py:9425-9468): one sequence of 5 tokens, blocks [0, 1] of 128 rows, 1026 cache rows
+    g = gen(970)
+    H, D = 32, 128
+    q = (torch.randn(1, H * D, generator=g) * 0.5).half().to(DEV)
+    k = (torch.randn(1026, H * D, generator=g) * 0.5).half().to(DEV)
+    v = (torch.randn(1026, H * D, generator=g) * 0.5).half().to(DEV)
+    table = torch.tensor([[0, 1]], dtype=torch.int32, device=DEV)
+    mask = torch.zeros(1, 1, 5, dtype=torch.bool, device=DEV)
+    out = F.paged_attention(q, k, v, mask, [5], H, H, D, table, 128)
+    ref = O.paged_attention(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), [5], H, H, D, table.cpu(), 128)
+    assert_close(out, ref, **TOL[torch.float16], what="paged_attention, reference case", mismatch_ratio=1e-3)
+
+    # a decode batch over a shuffled block pool: ragged lengths (one empty), grouped heads, int64 table, more sequences
+    # than one launch of the table kernel carries
+    for dtype, B, Hq, Hkv, bsz, maxlen in ((torch.float16, 70, 8, 2, 16, 700), (torch.bfloat16, 5, 4, 4, 128, 1500), (torch.float32, 3, 4, 2, 8, 50)):
+        D = 128 if dtype != torch.float32 else 64
+        nblk = (maxlen + bsz - 1) // bsz
+        lens = torch.randint(1, maxlen + 1, (B,), generator=g).tolist()
+        lens[1] = 0
+        lens[0] = maxlen
+        pool = B * nblk + 3
+        perm = torch.randperm(pool, generator=g)[:B * nblk].view(B, nblk)
+        table = perm.to(torch.int64 if dtype == torch.float16 else torch.int32).to(DEV)
+        q = (torch.randn(B, Hq * D, generator=g) * 0.5).to(dtype).to(DEV)
+        k = (torch.randn(pool * bsz, Hkv * D, generator=g) * 0.5).to(dtype).to(DEV)
+        v = (torch.randn(pool * bsz, Hkv * D, generator=g) * 0.5).to(dtype).to(DEV)
+        out = F.paged_attention(q, k, v, None, lens, Hq, Hkv, D, table, bsz)
+        exact = O.paged_attention(q.cpu(), k.cpu(), v.cpu(), None, lens, Hq, Hkv, D, table.cpu(), bsz, exact=True)
+        keep = [i for i in range(B) if lens[i] > 0]
+        assert_close(out[keep], exact[keep], **TOL[dtype], what=f"paged_attention {dtype}")
+    with pytest.raises(rt.DiopiException):
+        F.paged_attention(q, k, v, None, [9, 9, 9], Hq, Hkv, D, table[:, :1], bsz)  # 9 tokens do not fit one block of 8
+    with pytest.raises(rt.DiopiException):
+        F.paged_attention(q, k, v, None, [9, 9], Hq, Hkv, D, table, bsz)  # batch mismatch
+    zero = F.paged_attention(q, k, v, None, [0, 0, 0], Hq, Hkv, D, table, bsz)
+    assert float(zero.abs().max()) == 0.0
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)

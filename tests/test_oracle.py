@@ -532,3 +532,99 @@ def test_flash_attention_agrees_with_varlen_and_loops():
                     want = sum(w[j] * v[bi, j, h // 2] for j in range(last + 1)) / sum(w)
                     assert_close(out[bi, ti, h], want, 1e-12, 1e-12, "loops")
                     assert abs(float(lse[bi, h, ti]) - math.log(sum(w))) < 1e-12
+
+
+def test_prompt_flash_attention_is_context_attention_on_equal_sequences():
+    g = rng(81)
+    bs, L, H, D = 3, 7, 4, 16
+    q, k, v = (torch.randn(bs * L, H * D, generator=g, dtype=torch.float64) for _ in range(3))
+    got = O.prompt_flash_attention(q, k, v, None, [L] * bs, L, H, H, D, exact=True)
+    want = torch.zeros(bs * L, H, D, dtype=torch.float64)
+    O.context_attention(q.view(-1, H, D), k.view(-1, H, D), v.view(-1, H, D), want, torch.arange(0, bs * L, L), torch.full((bs,), L), L, exact=True)
+    assert_close(got.view(-1, H, D), want, 1e-12, 1e-12, "padded prompt attention vs the lightllm prefill statement")
+    for b in range(bs):  # the first row of a sequence sees only itself
+        assert_close(got[b * L], v[b * L], 1e-14, 1e-15, "first row")
+    # the dtype-faithful composition on the reference's case shape (diopi_configs.py:9383-9423) stays near the float64 value
+    q16, k16, v16 = ((torch.randn(4, 4096, generator=g) * 0.5).half() for _ in range(3))
+    mask = torch.tensor([[[False, True], [False, False]]] * 2)
+    a = O.prompt_flash_attention(q16, k16, v16, mask, [2, 2], 2, 32, 32, 128)
+    b = O.prompt_flash_attention(q16, k16, v16, mask, [2, 2], 2, 32, 32, 128, exact=True)
+    assert a.shape == (4, 4096) and a.dtype == torch.float16
+    assert_close(a.double(), b.double(), 1e-2, 1e-2, "fp16 composition vs float64")
+
+
+def test_prompt_flash_attention_python_loops_with_fewer_kv_heads():
+    g = rng(82)
+    bs, L, H, Hkv, D = 2, 5, 4, 2, 8
+    q = torch.randn(bs * L, H * D, generator=g, dtype=torch.float64)
+    k = torch.randn(bs * L, Hkv * D, generator=g, dtype=torch.float64)
+    v = torch.randn(bs * L, Hkv * D, generator=g, dtype=torch.float64)
+    got = O.prompt_flash_attention(q, k, v, None, [L, 3], L, H, Hkv, D, exact=True)  # a shorter actual length changes nothing
+    for b in range(bs):
+        for t in range(L):
+            for h in range(H):
+                hk = h // (H // Hkv)
+                qv = q[b * L + t, h * D:(h + 1) * D]
+                w = [math.exp(float(qv @ k[b * L + j, hk * D:(hk + 1) * D]) / math.sqrt(D)) for j in range(t + 1)]
+                want = sum(w[j] * v[b * L + j, hk * D:(hk + 1) * D] for j in range(t + 1)) / sum(w)
+                assert_close(got[b * L + t, h * D:(h + 1) * D], want, 1e-12, 1e-12, "loops")
+    # one key/value head: the statement's own broadcast (customized_test.py:775) gives the same numbers
+    k1, v1 = k[:, :D].contiguous(), v[:, :D].contiguous()
+    got1 = O.prompt_flash_attention(q, k1, v1, None, [L, L], L, H, 1, D, exact=True)
+    xq = q.view(bs, L, H, D).transpose(1, 2)
+    sc = torch.matmul(xq, k1.view(bs, L, 1, D).transpose(1, 2).transpose(2, 3)) / math.sqrt(D)
+    sc = sc.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), float("-inf")).softmax(-1)
+    want1 = torch.matmul(sc, v1.view(bs, L, 1, D).transpose(1, 2)).transpose(1, 2).reshape(bs * L, H * D)
+    assert_close(got1, want1, 1e-12, 1e-12, "broadcast single key/value head")
+
+
+def test_paged_attention_reference_case_and_block_tables():
+    g = rng(83)
+    # diopi_configs.py:9425-9468: one sequence of 5 tokens, 32 heads of 128, 1026 cache rows, blocks [0, 1] of 128 rows:
+    # the statement (customized_test.py:797-819) reads rows 0..4
+    H, D = 32, 128
+    q = (torch.randn(1, H * D, generator=g) * 0.5).half()
+    k = (torch.randn(1026, H * D, generator=g) * 0.5).half()
+    v = (torch.randn(1026, H * D, generator=g) * 0.5).half()
+    table = torch.tensor([[0, 1]], dtype=torch.int32)
+    mask = torch.zeros(1, 1, 5, dtype=torch.bool)
+    got = O.paged_attention(q, k, v, mask, [5], H, H, D, table, 128)
+    assert O.paged_rows(table, 0, 5, 128).tolist() == [0, 1, 2, 3, 4]
+    kk = k[:5].view(1, 5, H, D).transpose(1, 2)
+    logics = (torch.matmul(q.view(1, 1, H, D).transpose(1, 2)[0], kk.transpose(2, 3)) / math.sqrt(D)).reshape(H, 5)
+    want = torch.matmul(logics.softmax(-1).reshape(1, H, 1, 5), v[:5].view(1, 5, H, D).transpose(1, 2)).view(1, H * D)
+    assert torch.equal(got, want), "the statement's own arithmetic on rows 0..4"
+    ex = O.paged_attention(q, k, v, mask, [5], H, H, D, table, 128, exact=True)
+    assert_close(got.double(), ex.double(), 1e-2, 1e-2, "fp16 composition vs float64")
+
+    # shuffled block tables, several sequences, grouped heads: explicit loops in float64
+    B, H, Hkv, D, bsz = 3, 4, 2, 8, 4
+    lens = [6, 0, 9]
+    table = torch.tensor([[5, 2, 7], [1, 1, 1], [0, 6, 3]], dtype=torch.int64)
+    q = torch.randn(B, H * D, generator=g, dtype=torch.float64)
+    k = torch.randn(8 * bsz, Hkv * D, generator=g, dtype=torch.float64)
+    v = torch.randn(8 * bsz, Hkv * D, generator=g, dtype=torch.float64)
+    got = O.paged_attention(q, k, v, None, lens, H, Hkv, D, table, bsz, exact=True)
+    assert O.paged_rows(table, 0, 6, bsz).tolist() == [20, 21, 22, 23, 8, 9]
+    assert float(got[1].abs().max()) == 0.0
+    for i in (0, 2):
+        rows = [int(table[i, t // bsz]) * bsz + t % bsz for t in range(lens[i])]
+        for h in range(H):
+            hk = h // 2
+            w = [math.exp(float(q[i, h * D:(h + 1) * D] @ k[r, hk * D:(hk + 1) * D]) / math.sqrt(D)) for r in rows]
+            want = sum(wj * v[r, hk * D:(hk + 1) * D] for wj, r in zip(w, rows)) / sum(w)
+            assert_close(got[i, h * D:(h + 1) * D], want, 1e-12, 1e-12, "loops")
+
+    # the same numbers from the two lightllm decode statements on the expanded row table
+    maxlen = max(lens)
+    b_loc = torch.zeros(B, maxlen, dtype=torch.int64)
+    for i in range(B):
+        if lens[i]:
+            b_loc[i, maxlen - lens[i]:] = O.paged_rows(table, i, lens[i], bsz)
+    start = torch.tensor([0, 6, 6])
+    blen = torch.tensor(lens)
+    logits = torch.zeros(H, sum(lens), dtype=torch.float64)
+    O.token_attention(q.view(B, H, D), k.view(-1, Hkv, D), logits, b_loc, start, blen, maxlen, exact=True)
+    out = torch.zeros(B, H, D, dtype=torch.float64)
+    O.token_softmax_reducev(logits, v.view(-1, Hkv, D), out, b_loc, start, blen, maxlen, 0, exact=True)
+    assert_close(got.view(B, H, D), out, 1e-12, 1e-12, "paged attention vs token_attention + token_softmax_reducev")
