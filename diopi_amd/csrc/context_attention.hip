@@ -249,25 +249,33 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         kSrc[it] = r * rowBytes + (((lane % 16) ^ (r & 15)) * 16);
         vSrc[it] = r * rowBytes + (((lane % 16) ^ (4 * (r & 3))) * 16);
     }
-    // Requests tile jt into buffer jt & 1.  Unconditional: past the last tile it fetches the last tile again, into
-    // the buffer nobody reads any more.
-    auto requestTile = [&](int jt) {
-        const int jtL = jt < numKeyTiles ? jt : numKeyTiles - 1;
-        const int rowsLeft = L - jtL * kBN;
-        const int valid = rowsLeft < kBN ? rowsLeft : kBN;
-        const int bytes = static_cast<int>(((valid - 1) * rowPitch + kHD) * static_cast<int64_t>(sizeof(T)));
-        const uint64_t kAddr = reinterpret_cast<uint64_t>(kBase + jtL * kBN * rowPitch);
-        const uint64_t vAddr = reinterpret_cast<uint64_t>(vBase + jtL * kBN * rowPitch);
-        const u32x4 kBuf = {static_cast<uint32_t>(kAddr), static_cast<uint32_t>(kAddr >> 32) & 0xffffu, static_cast<uint32_t>(bytes), kRawBufferWord3};
-        const u32x4 vBuf = {static_cast<uint32_t>(vAddr), static_cast<uint32_t>(vAddr >> 32) & 0xffffu, static_cast<uint32_t>(bytes), kRawBufferWord3};
-        const uint32_t dst = ldsBase + (jt & 1) * kBufBytes + waveU * kChunks * 1024;
+    // Requests the next tile into the buffer the previous one left.  The scalar state (tile addresses, LDS address)
+    // advances from call to call so that a request costs a handful of scalar instructions; the last tile of a
+    // sequence gets a shorter descriptor (rows past the sequence read as zeros), tiles past the last are not requested.
+    const int64_t tileBytes = static_cast<int64_t>(kBN) * rowPitch * static_cast<int64_t>(sizeof(T));
+    const int fullBytes = static_cast<int>(((kBN - 1) * rowPitch + kHD) * static_cast<int64_t>(sizeof(T)));
+    const int lastBytes = static_cast<int>(((L - (numKeyTiles - 1) * kBN - 1) * rowPitch + kHD) * static_cast<int64_t>(sizeof(T)));
+    uint64_t kNext = reinterpret_cast<uint64_t>(kBase);
+    uint64_t vNext = reinterpret_cast<uint64_t>(vBase);
+    uint32_t dstNext = ldsBase + waveU * kChunks * 1024;
+    int nextTile = 0;
+    auto requestNext = [&]() {
+        if (nextTile < numKeyTiles) {  // wave-uniform
+            const uint32_t bytes = static_cast<uint32_t>(nextTile == numKeyTiles - 1 && L < numKeyTiles * kBN ? lastBytes : fullBytes);
+            const u32x4 kBuf = {static_cast<uint32_t>(kNext), static_cast<uint32_t>(kNext >> 32) & 0xffffu, bytes, kRawBufferWord3};
+            const u32x4 vBuf = {static_cast<uint32_t>(vNext), static_cast<uint32_t>(vNext >> 32) & 0xffffu, bytes, kRawBufferWord3};
 #pragma unroll
-        for (int it = 0; it < kChunks; ++it) {
-            loadToLds16(kBuf, dst + it * 1024, kSrc[it]);
-            loadToLds16(vBuf, dst + kTileBytes + it * 1024, vSrc[it]);
+            for (int it = 0; it < kChunks; ++it) {
+                loadToLds16(kBuf, dstNext + it * 1024, kSrc[it]);
+                loadToLds16(vBuf, dstNext + kTileBytes + it * 1024, vSrc[it]);
+            }
         }
+        kNext += tileBytes;
+        vNext += tileBytes;
+        dstNext ^= kBufBytes;
+        ++nextTile;
     };
-    requestTile(0);
+    requestNext();
     // ---- operand addresses inside a buffer ----
     // K (A operand of S^T): row 32 sb + n, packet 2 st + hh, one 16-byte read.
     // V^T (A operand of O^T): a lane needs 8 keys of one dim, which in the row-major V tile are 8 rows apart by 256
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         // every wave has left tile jt-1, whose buffer the request for tile jt+1 now fills while this tile is used.
         waitLdsLoads();
         __syncthreads();
-        requestTile(jt + 1);
+        requestNext();
         const LdsByte* sBuf = lds + (jt & 1) * kBufBytes;
 
         const int key0 = jt * kBN;
