@@ -32,6 +32,7 @@
 // second output.  That form is a template flag (GEN): the lightllm operator keeps its literal scale and its
 // compile-time causal structure.
 #include <cmath>
+#include <type_traits>
 
 #include "common.hpp"
 #include "device.hpp"
@@ -73,11 +74,22 @@ template <>
 struct Mfma32<half_t> {
     using Frag = f16x8;
     static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    // acc + lo + hi of a packed pair, in one instruction
+    static __device__ __forceinline__ float addPair(uint32_t pair, float acc) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 ones = {static_cast<_Float16>(1.f), static_cast<_Float16>(1.f)};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pair), ones, acc, false);
+    }
 };
 template <>
 struct Mfma32<bf16_t> {
     using Frag = bf16x8;
     static __device__ __forceinline__ f32x16 mma(Frag a, Frag b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ float addPair(uint32_t pair, float acc) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        const b2 ones = {static_cast<__bf16>(1.f), static_cast<__bf16>(1.f)};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, pair), ones, acc, false);
+    }
 };
 
 template <typename Frag>
@@ -97,6 +109,16 @@ __device__ __forceinline__ void loadToLds16(u32x4 rsrc, uint32_t ldsAddr, int by
 }
 #pragma clang diagnostic pop
 __device__ __forceinline__ void waitLdsLoads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// max(v, v of lane ^ 32) without a trip through the LDS crossbar: v_permlane32_swap exchanges the upper half of its
+// first operand with the lower half of its second, so two copies of v become (lower half twice, upper half twice).
+// The instruction is written out because the compiler's builtin returns the first result twice; the s_nop cover the
+// wait states the instruction needs next to vector instructions that write or read its operands.
+__device__ __forceinline__ float maxWithOtherHalf(float v) {
+    float lo = v, hi = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+    return fmaxf(lo, hi);
+}
 
 // Sequence geometry with every value forced inside the tensors.
 struct SeqInfo {
@@ -203,6 +225,11 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(kvHead) * kHD;
 
     // ---- Q fragments (B operand of S^T): row = m0 + 32*wave + n, k slot (hh, e) <-> dim 16*s + 8*hh + e ----
+    // fp16: the query is multiplied by softmax_scale * log2(e) here, once, so that the first product delivers the
+    // exponent of 2 directly.  That rounds the scaled query to 11 bits, the size of the rounding the reference applies
+    // to its fp16 scores; bf16 (8 bits) keeps the multiplication in fp32, one instruction per score.
+    constexpr bool kFold = std::is_same<T, half_t>::value;
+    const float toLog2 = kFold ? 1.f : scaleLog2;  // from the unit of the score accumulators to powers of two
     const int qRow = m0 + wave * 32 + n;
     const int qRowLd = qRow < L ? qRow : L - 1;
     Frag qf[kHD / 16];
@@ -210,7 +237,12 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     for (int s = 0; s < kHD / 16; ++s) {
         FragBits<Frag> u;
         u.raw = *reinterpret_cast<const u32x4*>(qBase + qRowLd * qPitch + s * 16 + hh * 8);
-        qf[s] = u.f;
+        if constexpr (kFold) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<T>(static_cast<float>(u.f[e]) * scaleLog2);
+        } else {
+            qf[s] = u.f;
+        }
     }
 
     f32x16 o[kHD / 32];
@@ -219,7 +251,13 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[mb][r] = 0.f;
     }
-    float mRun = -1e30f;
+    // Reference maximum of this lane's query row in the unit of the score accumulators, and its negative in all 16
+    // registers of an accumulator tuple: the first product of a tile starts from it, so the scores arrive as
+    // (score - reference), ready for the exponential.
+    float mRun = 0.f;
+    f32x16 negRef;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negRef[r] = 0.f;
     float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
 
     const int kEnd = (causal && m0 + BM < L) ? m0 + BM : L;  // keys 0 .. kEnd-1 are visible to this tile
@@ -317,11 +355,8 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
         // alternate so that consecutive products never wait on each other's accumulator.
         f32x16 s[2];
-#pragma unroll
-        for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[sb][r] = 0.f;
-        }
+        s[0] = negRef;
+        s[1] = negRef;
         constexpr int kKDepth = 2;  // K operand steps in flight: LDS latency under load spans several products
         FragBits<Frag> kf[kKDepth][2];
         auto loadK = [&](int st, int b) {
@@ -368,40 +403,59 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
                 }
             }
         }
-        float tmax = -1e30f;
+        // largest score of the tile relative to the reference: four independent chains, then the other lane half
+        float tm[4];
 #pragma unroll
-        for (int sb = 0; sb < 2; ++sb) {
+        for (int c = 0; c < 4; ++c) {
+            tm[c] = fmaxf(s[c / 2][8 * (c % 2)], s[c / 2][8 * (c % 2) + 1]);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[sb][r]);
+            for (int r = 2; r < 8; ++r) tm[c] = fmaxf(tm[c], s[c / 2][8 * (c % 2) + r]);
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-        // The reference maximum only follows the true one when it has fallen behind by more than 2^kLazyLog2 (a
-        // wave-uniform, rarely taken branch after the first tiles): probabilities then reach at most 2^kLazyLog2,
-        // which the 16-bit types hold with full relative precision, and the accumulators are rescaled only then.
-        if (__any((tmax - mRun) * scaleLog2 > kLazyLog2)) {
-            const float mNew = fmaxf(mRun, tmax);
-            const float alpha = __builtin_amdgcn_exp2f((mRun - mNew) * scaleLog2);
-            mRun = mNew;
+        const float tmax = maxWithOtherHalf(fmaxf(fmaxf(tm[0], tm[1]), fmaxf(tm[2], tm[3])));
+        // The reference only follows the true maximum when it has fallen behind by more than 2^kLazyLog2 (a
+        // wave-uniform, rarely taken branch after the first tile, where it is set for the first time): probabilities
+        // then reach at most 2^kLazyLog2, which the 16-bit types hold with full relative precision, and the
+        // accumulators are rescaled only then.
+        if (jt == 0 || __any(tmax * toLog2 > kLazyLog2)) {
+            const float up = jt == 0 ? tmax : fmaxf(tmax, 0.f);
+            const float alpha = __builtin_amdgcn_exp2f(-up * toLog2);
+            mRun += up;
             lRun *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) negRef[r] = -mRun;
 #pragma unroll
             for (int mb = 0; mb < kHD / 32; ++mb) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) o[mb][r] *= alpha;
             }
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[sb][r] -= up;
+            }
         }
-        const float mc = mRun * scaleLog2;
         float psum[4] = {0.f, 0.f, 0.f, 0.f};
         Frag pf[2][2];
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
+                FragBits<Frag> pk;
+                if constexpr (kFold) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2 - mc);
-                    psum[j & 3] += p;
-                    pf[sb][u][j] = static_cast<T>(p);
+                    for (int j = 0; j < 8; ++j) pk.f[j] = static_cast<T>(__builtin_amdgcn_exp2f(s[sb][u * 8 + j]));
+                    // the row sum takes the rounded probabilities (the ones the second product multiplies), two per instruction
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) psum[w] = Ops::addPair(pk.raw[w], psum[w]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2);
+                        psum[j & 3] += p;
+                        pk.f[j] = static_cast<T>(p);
+                    }
                 }
+                pf[sb][u] = pk.f;
             }
         }
         lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
@@ -423,7 +477,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     if constexpr (GEN) {
         // ln sum_j exp(scale * s_j) = ln 2 * (reference maximum in log2 units + log2 of the sum relative to it)
         if (a.lse != nullptr && hh == 0 && qRow < L && qRow < a.lseStride)
-            a.lse[(static_cast<int64_t>(planned.x) * a.H + head) * a.lseStride + qRow] = 0.6931471805599453f * (mRun * scaleLog2 + __builtin_amdgcn_logf(lTot));
+            a.lse[(static_cast<int64_t>(planned.x) * a.H + head) * a.lseStride + qRow] = 0.6931471805599453f * (mRun * toLog2 + __builtin_amdgcn_logf(lTot));
     }
     waitLdsLoads();
     __syncthreads();  // the K/V tiles are dead (and the surplus request has landed); reuse the storage as a [BM][kLD] output tile
