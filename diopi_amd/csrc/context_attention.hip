@@ -345,26 +345,29 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         // every wave has left tile jt-1, whose buffer the request for tile jt+1 now fills while this tile is used.
         waitLdsLoads();
         __syncthreads();
-        requestNext();
         const LdsByte* sBuf = lds + (jt & 1) * kBufBytes;
-
         const int key0 = jt * kBN;
-        if (causal && key0 > waveRowHi) continue;  // entirely above the diagonal for this wave (barriers are at the loop top)
+        const bool skip = causal && key0 > waveRowHi;  // entirely above the diagonal for this wave
 
         // ---- S^T = K . Q^T for the two 32-key blocks ----
         // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
-        // alternate so that consecutive products never wait on each other's accumulator.
-        f32x16 s[2];
-        s[0] = negRef;
-        s[1] = negRef;
+        // alternate so that consecutive products never wait on each other's accumulator.  The first operands are
+        // requested before the scalar work of the tile request, which then runs while they travel.
         constexpr int kKDepth = 2;  // K operand steps in flight: LDS latency under load spans several products
         FragBits<Frag> kf[kKDepth][2];
         auto loadK = [&](int st, int b) {
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb) kf[b][sb].raw = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(sBuf + kOff[st] + sb * 32 * 256);
         };
+        if (!skip) {
 #pragma unroll
-        for (int st = 0; st < kKDepth - 1; ++st) loadK(st, st);
+            for (int st = 0; st < kKDepth - 1; ++st) loadK(st, st);
+        }
+        requestNext();
+        if (skip) continue;  // barriers are at the loop top
+        f32x16 s[2];
+        s[0] = negRef;
+        s[1] = negRef;
 #pragma unroll
         for (int st = 0; st < kHD / 16; ++st) {
             if (st + kKDepth - 1 < kHD / 16) loadK(st + kKDepth - 1, (st + kKDepth - 1) % kKDepth);
@@ -434,41 +437,36 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
                 for (int r = 0; r < 16; ++r) s[sb][r] -= up;
             }
         }
+        // ---- probabilities and O^T += V^T . P^T, one group of 16 keys at a time ----
+        // k slot (hh, j) of group g = 2*sb + u is key 16*g + 8*(j/4) + 4*hh + j%4; accumulator row n' of o[mb] stands
+        // for dim 32*mb + n'.  The exponentials of a group are issued right before its four products, so that they run
+        // while the matrix pipe works on the previous group's (of this wave and of the other wave of the SIMD).
         float psum[4] = {0.f, 0.f, 0.f, 0.f};
-        Frag pf[2][2];
-#pragma unroll
-        for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                FragBits<Frag> pk;
-                if constexpr (kFold) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) pk.f[j] = static_cast<T>(__builtin_amdgcn_exp2f(s[sb][u * 8 + j]));
-                    // the row sum takes the rounded probabilities (the ones the second product multiplies), two per instruction
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) psum[w] = Ops::addPair(pk.raw[w], psum[w]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2);
-                        psum[j & 3] += p;
-                        pk.f[j] = static_cast<T>(p);
-                    }
-                }
-                pf[sb][u] = pk.f;
-            }
-        }
-        lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
-        // ---- O^T += V^T . P^T : k slot (hh, j) of group g = 2*sb + u is key 16*g + 8*(j/4) + 4*hh + j%4 ----
-        // accumulator row n' of o[mb] stands for dim 32*mb + n'
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+            const int sb = g / 2, u = g % 2;
+            FragBits<Frag> pk;
+            if constexpr (kFold) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) pk.f[j] = static_cast<T>(__builtin_amdgcn_exp2f(s[sb][u * 8 + j]));
+                // the row sum takes the rounded probabilities (the ones the second product multiplies), two per instruction
+#pragma unroll
+                for (int w = 0; w < 4; ++w) psum[w] = Ops::addPair(pk.raw[w], psum[w]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float p = __builtin_amdgcn_exp2f(s[sb][u * 8 + j] * scaleLog2);
+                    psum[j & 3] += p;
+                    pk.f[j] = static_cast<T>(p);
+                }
+            }
             if (g + 1 < 4) loadV(g + 1, (g + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pf[g / 2][g % 2], o[mb]);
+            for (int mb = 0; mb < kHD / 32; ++mb) o[mb] = Ops::mma(vf[g & 1][mb].f, pk.f, o[mb]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        lRun += (psum[0] + psum[1]) + (psum[2] + psum[3]);
     }
 
     // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
