@@ -225,10 +225,12 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     const T* vBase = v + si.start * rowPitch + static_cast<int64_t>(kvHead) * kHD;
 
     // ---- Q fragments (B operand of S^T): row = m0 + 32*wave + n, k slot (hh, e) <-> dim 16*s + 8*hh + e ----
-    // fp16: the query is multiplied by softmax_scale * log2(e) here, once, so that the first product delivers the
-    // exponent of 2 directly.  That rounds the scaled query to 11 bits, the size of the rounding the reference applies
-    // to its fp16 scores; bf16 (8 bits) keeps the multiplication in fp32, one instruction per score.
-    constexpr bool kFold = std::is_same<T, half_t>::value;
+    // The query is multiplied by softmax_scale * log2(e) here, once, so that the first product delivers the exponent
+    // of 2 directly.  That rounds the scaled query to the element type, the size of the rounding the reference applies
+    // to its scores (functions_lightllm.cpp:121 keeps them in the tensor dtype).  The general form with bf16 tensors
+    // (8 bits) does not: it also returns the log-sum-exp, which would inherit that rounding; it keeps the
+    // multiplication in fp32, one instruction per score, and sums the unrounded probabilities.
+    constexpr bool kFold = std::is_same<T, half_t>::value || !GEN;
     const float toLog2 = kFold ? 1.f : scaleLog2;  // from the unit of the score accumulators to powers of two
     const int qRow = m0 + wave * 32 + n;
     const int qRowLd = qRow < L ? qRow : L - 1;
