@@ -394,7 +394,18 @@ def main():
         ms_f = timed(fav)
         record("diopiFlashAttentionVarLen (causal, 32 heads over 8 kv heads, lse)", f"cfg4 tokens fp16 B=8 T={w4['T']}", ms_f, flops, "mfma", "f16", None,
                note="widening beyond the seven hot-path operators; the prefill kernel in its general form")
-        del w4, hf, k8, v8, lse
+        # the lightllm operator once more with bf16 tensors (same tokens, same flop count)
+        qb, kb, vb = (w4[k].to(torch.bfloat16) for k in ("q", "k", "v"))
+        ob = torch.zeros_like(qb)
+        hb = {k: Tensor(v) for k, v in dict(q=qb, k=kb, v=vb, o=ob).items()}
+
+        def pre_bf16(i):
+            check(impl.diopiContextAttentionInference(ctx.handle, hb["o"].handle, hb["q"].handle, hb["k"].handle, hb["v"].handle, h["b_start_loc"].handle,
+                                                      h["b_seq_len"].handle, w4["max_input_len"]), "diopiContextAttentionInference")
+
+        ms_b = timed(pre_bf16)
+        record("diopiContextAttentionInference", f"cfg4 tokens in bf16 B=8 T={w4['T']}", ms_b, flops, "mfma", "bf16", None)
+        del w4, hf, k8, v8, lse, hb, qb, kb, vb, ob
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ the JSON line
