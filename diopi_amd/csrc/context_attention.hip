@@ -11,16 +11,17 @@
 // are not written; max_input_len is not needed (the reference never reads it either).
 //
 // MFMA kernel (fp16 / bf16, D == 128).  A work-group of 4 or 8 waves owns 128 or 256 query rows of one
-// (sequence, head); each wave owns 32 of them.  Key/value tiles of 64 rows are staged in LDS (two buffers, one
-// barrier per tile, the global request for a tile is issued a whole iteration before it is needed) and shared by
-// the waves.  Everything is computed transposed so that no cross-lane data movement is needed between the two
-// matrix products:
+// (sequence, head); each wave owns 32 of them.  Key/value tiles of 64 rows are fetched into LDS by 16-byte buffer
+// loads that write LDS directly (two buffers, one barrier per tile, a tile is requested a whole iteration before it is
+// needed; packets XOR-swizzled by row so that every operand read is free of bank conflicts) and shared by the waves.
+// Everything is computed transposed so that no cross-lane data movement is needed between the two matrix products:
 //   S^T[key, q]  = K[key, :] . Q[q, :]      v_mfma_f32_32x32x16, A = K rows from LDS, B = Q rows (registers)
-//   O^T[d, q]   += V^T[d, key] . P^T[key, q]                    A = V^T rows from LDS, B = P^T
+//   O^T[d, q]   += V^T[d, key] . P^T[key, q]                    A = V^T gathered from the row-major V tile, B = P^T
 // In the 32x32 accumulator layout a lane holds one query column, so the row maximum, the row sum and the rescaling
 // of O^T are per-lane scalars (one exchange with lane ^ 32 per tile), and the exponentiated scores are already in
-// the B-operand layout of the second product.  The V tile is transposed once, when it is staged (byte permutes on
-// key pairs, dword writes), so that the second product's A operand is a single 16-byte LDS read like the first's.
+// the B-operand layout of the second product.  The V^T operand comes from transposing LDS reads (ds_read_b64_tr_b16),
+// two per matrix instruction.  The first product starts from the negative reference maximum and, where the scale is
+// folded into the query fragments, delivers the argument of the exponential directly.
 // The softmax reference maximum is updated lazily (only when it lags by more than 2^8), which keeps the rescaling
 // of the 64 accumulator registers out of the common path.
 // Work-groups are numbered so that the query tiles of one head land on the same XCD (they share that head's K/V
@@ -396,8 +397,8 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         __builtin_amdgcn_sched_barrier(0);
         // accumulator register r of block sb holds key  key0 + 32*sb + 8*(r/4) + 4*hh + r%4  for query row qRow
         if (causal ? key0 + kBN - 1 > waveRowLo : key0 + kBN > L) {
-            // causal: keys past the query's own position (which covers keys past the sequence, staged as copies of its
-            // last row); full attention: only those
+            // causal: keys past the query's own position (which covers keys past the sequence, which arrive as
+            // zeros); full attention: only those
             const int lastKey = causal ? qRow : L - 1;
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb) {
