@@ -481,7 +481,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
             a.lse[(static_cast<int64_t>(planned.x) * a.H + head) * a.lseStride + qRow] = 0.6931471805599453f * (mRun * toLog2 + __builtin_amdgcn_logf(lTot));
     }
     waitLdsLoads();
-    __syncthreads();  // the K/V tiles are dead (and the surplus request has landed); reuse the storage as a [BM][kLD] output tile
+    __syncthreads();  // the K/V tiles are dead and no request is in flight; reuse the storage as a [BM][kLD] output tile
     T* sO = smem;
     static_assert(kHD == 128, "scaleLog2 is written out for head size 128");
 #pragma unroll
