@@ -56,7 +56,7 @@ struct CtxArgs {
     int batch;
     int H;
     int64_t rows;      // rows of q / k / v / out
-    const int2* plan;  // [tilesBound] visiting order of the query tiles of one head, written by ctxAttnPlan
+    const int4* plan;  // [tilesBound] visiting order of the query tiles of one head, written by ctxAttnPlan
     int tilesBound;    // upper bound on the number of 128-row query tiles over all sequences
     int totalItems;    // H * tilesBound
     // general form only (diopiFlashAttentionVarLen); the lightllm operator leaves these at their defaults
@@ -142,18 +142,25 @@ __device__ __forceinline__ SeqInfo loadSeq(const CtxArgs& a, int i) {
     return s;
 }
 
-// Visiting order of the query tiles of one head: entry p of `plan` is (sequence, query tile index), sorted by tile
+// Visiting order of the query tiles of one head: entry p of `plan` is (sequence, query tile index, first row and
+// length of the sequence: everything a work-group needs, in one load), sorted by tile
 // index descending.  A query tile with index t attends to t + 1 key blocks, so this is longest-job-first and the
 // short tiles fill the tail of the launch whatever the mix of sequence lengths.  With the sequences ranked by tile
 // count (descending), the sequences that own a tile of index t are a prefix of that ranking, hence
 //   position(seq, t) = sum_s max(0, tiles_s - 1 - t)  +  rank(seq).
 // One work-group; tile counts are kept in LDS.  Unused entries (the bound over-counts) get sequence -1.
 constexpr int kPlanThreads = 1024;
-__global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ plan, CtxArgs a, int maxTiles, int bm) {
-    extern __shared__ int sTiles[];  // [batch]
+__global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int4* __restrict__ plan, CtxArgs a, int maxTiles, int bm) {
+    extern __shared__ int sTiles[];  // [batch] tile counts, [batch] ranks, [maxTiles] offsets, [2 * batch] geometry
     const int tid = threadIdx.x;
-    for (int s = tid; s < a.batch; s += kPlanThreads) sTiles[s] = static_cast<int>((loadSeq(a, s).len + bm - 1) / bm);
-    for (int p = tid; p < a.tilesBound; p += kPlanThreads) plan[p] = make_int2(-1, 0);
+    int* sStart = sTiles + 2 * a.batch + maxTiles;  // [batch] first row, then [batch] length (the launcher checked that row counts fit 32 bits)
+    for (int s = tid; s < a.batch; s += kPlanThreads) {
+        const SeqInfo si = loadSeq(a, s);
+        sTiles[s] = static_cast<int>((si.len + bm - 1) / bm);
+        sStart[s] = static_cast<int>(si.start);
+        sStart[a.batch + s] = static_cast<int>(si.len);
+    }
+    for (int p = tid; p < a.tilesBound; p += kPlanThreads) plan[p] = make_int4(-1, 0, 0, 0);
     __syncthreads();
     for (int s = tid; s < a.batch; s += kPlanThreads) {
         const int nt = sTiles[s];
@@ -181,7 +188,7 @@ __global__ __launch_bounds__(kPlanThreads) void ctxAttnPlan(int2* __restrict__ p
         for (int t = tid; t < nt; t += kPlanThreads) {
             // overlapping sequences (a caller error) could count more tiles than the bound the table is sized for
             const int pos = (t < maxTiles ? sTiles[2 * a.batch + t] : a.tilesBound) + rank;
-            if (pos < a.tilesBound) plan[pos] = make_int2(s, t);
+            if (pos < a.tilesBound) plan[pos] = make_int4(s, t, sStart[s], sStart[a.batch + s]);
         }
     }
 }
@@ -206,10 +213,12 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     if (item >= a.totalItems) return;
     const int head = item / a.tilesBound;
     const int tileFlat = item % a.tilesBound;
-    const int2 planned = a.plan[tileFlat];  // (sequence, query tile), longest tiles first; sequence -1 = padding
+    const int4 planned = a.plan[tileFlat];  // (sequence, query tile, first row, length), longest tiles first; sequence -1 = padding
     if (planned.x < 0) return;
     const int qt = planned.y;
-    const SeqInfo si = loadSeq(a, planned.x);
+    SeqInfo si;
+    si.start = planned.z;
+    si.len = planned.w;
     const int L = static_cast<int>(si.len);              // the launcher checked that row counts fit 32 bits
     const int m0 = qt * BM;
 
@@ -581,11 +590,11 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     a.totalItems = static_cast<int>(total);
     // visiting order of the query tiles (context-owned scratch, rebuilt by every call on the device)
     void* planMem = nullptr;
-    ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int2), &planMem));
-    a.plan = static_cast<const int2*>(planMem);
+    ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int4), &planMem));
+    a.plan = static_cast<const int4*>(planMem);
     const int maxTiles = static_cast<int>(ceilDiv(a.rows, BM));
-    const size_t planLds = (2 * static_cast<size_t>(a.batch) + maxTiles) * sizeof(int);
-    hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int2*>(planMem), a, maxTiles, BM);
+    const size_t planLds = (4 * static_cast<size_t>(a.batch) + maxTiles) * sizeof(int);
+    hipLaunchKernelGGL(ctxAttnPlan, dim3(1), dim3(kPlanThreads), planLds, stream, static_cast<int4*>(planMem), a, maxTiles, BM);
     ROCM_LAUNCH_CHECK();
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
     constexpr int kStaging = 2 * 2 * kBN * kHD, kOutTile = BM * kLD;  // elements: two (K, V) buffers; the output tile that reuses them
@@ -620,7 +629,7 @@ diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, con
     const bool aligned =
         ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
     // the planning kernel keeps two ints per sequence and one per query tile in LDS
-    const bool planFits = (2 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
+    const bool planFits = (4 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
     // the tile requests address a 64-row tile with 32-bit byte offsets
     const bool tileFits = static_cast<int64_t>(a.H) * kHD * 8 * kBN < INT32_MAX;
     const bool fast = D == kHD && aligned && planFits && tileFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
