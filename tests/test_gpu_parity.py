@@ -825,6 +825,34 @@ def test_paged_attention_reference_case_and_block_tables():
     assert float(zero.abs().max()) == 0.0
 
 
+def test_paged_attention_full_size_equals_the_two_decode_operators():
+    # benchmark size (64 sequences of 512..2048 tokens, 32 heads of 128, 1024 blocks of 128 rows): the block table expanded
+    # on the host into the row table of the lightllm operators must give the same bits, since the same kernels run
+    g = gen(980)
+    B, H, D, bsz, nblk = 64, 32, 128, 128, 16
+    lens = torch.randint(512, 2049, (B,), generator=g)
+    table = torch.randperm(B * nblk, generator=g).view(B, nblk).int()
+    q = (torch.randn(B, H * D, generator=g) * 0.5).half().to(DEV)
+    k = (torch.randn(B * nblk * bsz, H * D, generator=g) * 0.5).half().to(DEV)
+    v = (torch.randn(B * nblk * bsz, H * D, generator=g) * 0.5).half().to(DEV)
+    out = F.paged_attention(q, k, v, None, lens.tolist(), H, H, D, table.to(DEV), bsz)
+    maxlen = int(lens.max())
+    b_loc = torch.zeros(B, maxlen, dtype=torch.int32)
+    for i in range(B):
+        L = int(lens[i])
+        b_loc[i, maxlen - L:] = O.paged_rows(table, i, L, bsz).int()
+    start = (torch.cumsum(lens, 0) - lens).int()
+    logits = torch.zeros(H, int(lens.sum()), dtype=torch.float16, device=DEV)
+    F.token_attention(q.view(B, H, D), k.view(-1, H, D), logits, b_loc.to(DEV), start.to(DEV), lens.int().to(DEV), maxlen)
+    want = torch.zeros(B, H, D, dtype=torch.float16, device=DEV)
+    F.token_softmax_reducev(logits, v.view(-1, H, D), want, b_loc.to(DEV), start.to(DEV), lens.int().to(DEV), maxlen, 0)
+    assert_bit_equal(out.view(B, H, D), want, "paged attention vs token attention + softmax-reduce-v on the expanded table")
+    # and a sampled sequence against the float64 oracle
+    i = 7
+    exact = O.paged_attention(q[i:i + 1].cpu(), k.cpu(), v.cpu(), None, [int(lens[i])], H, H, D, table[i:i + 1], bsz, exact=True)
+    assert_close(out[i:i + 1], exact, **TOL[torch.float16], what="paged attention, sampled sequence vs float64")
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
