@@ -825,6 +825,26 @@ def test_paged_attention_reference_case_and_block_tables():
     assert float(zero.abs().max()) == 0.0
 
 
+def test_prompt_flash_attention_full_size_matches_context_attention():
+    # 8 prompts of 2048 rows, 32 heads of 128 (the prefill benchmark's head geometry): the padded-batch operator and
+    # the lightllm operator on the same rows cut into equal sequences are two entries over one kernel
+    g = gen(975)
+    bs, L, H, D = 8, 2048, 32, 128
+    q, k, v = ((torch.randn(bs * L, H * D, generator=g) * 0.5).half().to(DEV) for _ in range(3))
+    out = F.prompt_flash_attention(q, k, v, None, [L] * bs, L, H, H, D)
+    want = torch.zeros(bs * L, H, D, dtype=torch.float16, device=DEV)
+    start = torch.arange(0, bs * L, L, dtype=torch.int32, device=DEV)
+    F.context_attention(q.view(-1, H, D), k.view(-1, H, D), v.view(-1, H, D), want, start, torch.full((bs,), L, dtype=torch.int32, device=DEV), L)
+    assert_close(out.view(-1, H, D), want, rtol=2e-3, atol=2e-4, what="prompt_flash_attention vs context_attention at full size")
+    # size-independent properties: the first row of a sequence is its value row; rows of sampled (sequence, head) pairs against float64
+    assert torch.equal(out[3 * L].cpu(), v[3 * L].cpu())
+    for b, h in ((0, 0), (5, 17)):
+        rows = slice(b * L, b * L + 300)
+        cols = slice(h * D, (h + 1) * D)
+        exact = O.prompt_flash_attention(q[rows, cols].cpu(), k[rows, cols].cpu(), v[rows, cols].cpu(), None, [300], 300, 1, 1, D, exact=True)
+        assert_close(out[rows, cols], exact, **TOL[torch.float16], what="prompt_flash_attention, sampled rows vs float64")
+
+
 def test_paged_attention_full_size_equals_the_two_decode_operators():
     # benchmark size (64 sequences of 512..2048 tokens, 32 heads of 128, 1024 blocks of 128 rows): the block table expanded
     # on the host into the row table of the lightllm operators must give the same bits, since the same kernels run
