@@ -873,6 +873,83 @@ def test_paged_attention_full_size_equals_the_two_decode_operators():
     assert_close(out[i:i + 1], exact, **TOL[torch.float16], what="paged attention, sampled sequence vs float64")
 
 
+# ----------------------------------------------------------------------------- base pointers that are not 16-byte aligned
+def _off(t: torch.Tensor) -> torch.Tensor:
+    """The same values in a dense device tensor whose first element sits one element past an aligned allocation."""
+    flat = torch.empty(t.numel() + 1, dtype=t.dtype, device=DEV)
+    view = flat[1:].view(t.shape)
+    view.copy_(t)
+    assert view.is_contiguous() and view.data_ptr() % 16 != 0
+    return view
+
+
+def test_unaligned_base_pointers_take_the_slow_paths_and_stay_correct():
+    # a framework may hand over dense views that start in the middle of an allocation: every operator must either
+    # use narrower accesses or its general kernel, never a wrong fast path
+    g = gen(990)
+    dt = torch.float16
+    tol = TOL[dt]
+    # RMSNorm forward and backward
+    x, wgt, go = (torch.randn(64, 512, generator=g) * 0.5).to(dt), torch.randn(512, generator=g).to(dt), (torch.randn(64, 512, generator=g) * 0.5).to(dt)
+    xd, wd, god = _off(x), _off(wgt), _off(go)
+    out = F.rms_norm(xd, (512,), wd, None, 1e-6)
+    inv = F.GLOBAL_STATE["rms_norm_inv_rms"]
+    r_out, r_inv = O.rms_norm(x, (512,), wgt, None, 1e-6, exact=True)
+    assert_close(out, r_out, what="rms_norm, unaligned", **tol)
+    grads = F.rms_norm_backward([god], xd, wd, None, (512,), 1e-6, inv_rms=inv)
+    r_gi, r_gw, _ = O.rms_norm_backward(go, x, wgt, inv.cpu(), (512,), exact=True)
+    assert_close(grads["input"], r_gi, what="rms_norm_backward grad_input, unaligned", **tol)
+    assert_close(grads["weight"], r_gw, rtol=2e-2, atol=2e-2, what="rms_norm_backward grad_weight, unaligned")
+    # rotary, both forms
+    T, H, D = 33, 4, 128
+    q, k = (torch.randn(T, H, D, generator=g) * 0.5).to(dt), (torch.randn(T, H, D, generator=g) * 0.5).to(dt)
+    ang = torch.rand(T, 1, D // 2, generator=g) * 6.28
+    cos, sin = ang.cos().to(dt), ang.sin().to(dt)
+    rot = F.rotary_emb(_off(q), _off(cos), _off(sin), False, False)
+    assert_close(rot, O.rotary_emb(q, cos, sin, False, exact=True), what="rotary_emb, unaligned", **tol)
+    cos2, sin2 = torch.cat((cos, cos), -1).reshape(T, D), torch.cat((sin, sin), -1).reshape(T, D)
+    q2, k2 = _off(q.reshape(T, H * D)), _off(k.reshape(T, H * D))
+    rq, rk = O.rotary_emb_v2(q.reshape(T, H * D).clone(), k.reshape(T, H * D).clone(), cos2, sin2, D, exact=True)
+    F.rotary_emb_v2(q2, k2, _off(cos2), _off(sin2), D)
+    assert_close(q2, rq, what="rotary_emb_v2 query, unaligned", **tol)
+    assert_close(k2, rk, what="rotary_emb_v2 key, unaligned", **tol)
+    # scatter into the cache
+    cache = (torch.randn(96, H, D, generator=g)).to(dt)
+    dest = torch.randperm(96, generator=g)[:T].int()
+    cd = _off(cache)
+    F.destindex_copy_kv(_off(q), dest.to(DEV), cd)
+    assert_bit_equal(cd, O.destindex_copy_kv(q, dest, cache.clone()), "destindex_copy_kv, unaligned")
+    # decode
+    B, L = 3, 40
+    lens = torch.tensor([40, 17, 1], dtype=torch.int32)
+    b_loc = torch.stack([torch.randperm(96, generator=g)[:L] for _ in range(B)]).int()
+    start = (torch.cumsum(lens, 0) - lens).int()
+    qd = (torch.randn(B, H, D, generator=g) * 0.5).to(dt)
+    vc = (torch.randn(96, H, D, generator=g) * 0.5).to(dt)
+    logits = _off(torch.zeros(H, int(lens.sum()), dtype=dt))
+    F.token_attention(_off(qd), cd, logits, b_loc.to(DEV), start.to(DEV), lens.to(DEV), L)
+    ref_logits = torch.zeros(H, int(lens.sum()), dtype=torch.float64)
+    O.token_attention(qd, cd.cpu(), ref_logits, b_loc, start, lens, L, exact=True)
+    assert_close(logits, ref_logits, what="token_attention, unaligned", **tol)
+    dec = _off(torch.zeros(B, H, D, dtype=dt))
+    F.token_softmax_reducev(logits, _off(vc), dec, b_loc.to(DEV), start.to(DEV), lens.to(DEV), L, 0)
+    ref_dec = torch.zeros(B, H, D, dtype=torch.float64)
+    O.token_softmax_reducev(logits.cpu(), vc, ref_dec, b_loc, start, lens, L, 0, exact=True)
+    assert_close(dec, ref_dec, what="token_softmax_reducev, unaligned", **tol)
+    # prefill, both interfaces
+    Ls = torch.tensor([150, 70], dtype=torch.int32)
+    st = torch.tensor([0, 150], dtype=torch.int32)
+    pq, pk, pv = ((torch.randn(220, H, D, generator=g) * 0.5).to(dt) for _ in range(3))
+    po = _off(torch.zeros(220, H, D, dtype=dt))
+    F.context_attention(_off(pq), _off(pk), _off(pv), po, st.to(DEV), Ls.to(DEV), 150)
+    ref = torch.zeros(220, H, D, dtype=torch.float64)
+    O.context_attention(pq, pk, pv, ref, st, Ls, 150, exact=True)
+    assert_close(po, ref, what="context_attention, unaligned", **tol)
+    cu = torch.tensor([0, 150, 220], dtype=torch.int32)
+    fa = F.flash_attention_varlen(_off(pq), _off(pk), _off(pv), cu.to(DEV), cu.to(DEV), None, 150, 150, 0, None, True)
+    assert_close(fa, ref, what="flash_attention_varlen, unaligned", **tol)
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
