@@ -1018,6 +1018,52 @@ def test_two_threads_with_their_own_contexts_and_streams():
                 assert_bit_equal(got, want, f"thread {i}: {name}")
 
 
+# ----------------------------------------------------------------------------- a decode step recorded in a HIP graph
+def test_decode_step_in_a_hip_graph_replays_like_eager():
+    # serving loops record the decode step once and replay it: scatter of the new K/V rows, score rows, softmax and
+    # product with V.  Every launch goes to the context's stream and the scratch comes from the context's pool, so the
+    # step must be capturable after one eager run, and every replay must give what the eager call gives on the same inputs.
+    w = W.cfg3(DEV, seed=77, scale=1 / 8)
+    H, total, mil = w["H"], w["total_len"], w["max_input_len"]
+    stream = torch.cuda.Stream()
+    ctx = rt.Context(stream=stream)
+    logits = torch.zeros(H, total, dtype=torch.float16, device=DEV)
+    out = torch.zeros_like(w["q"])
+
+    def step():
+        F.destindex_copy_kv(w["new_k"], w["dest_loc"], w["k_cache"], ctx=ctx)
+        F.destindex_copy_kv(w["new_v"], w["dest_loc"], w["v_cache"], ctx=ctx)
+        F.token_attention(w["q"], w["k_cache"], logits, w["b_loc"], w["b_start_loc"], w["b_seq_len"], mil, ctx=ctx)
+        F.token_softmax_reducev(logits, w["v_cache"], out, w["b_loc"], w["b_start_loc"], w["b_seq_len"], mil, 0, ctx=ctx)
+
+    with torch.cuda.stream(stream):
+        step()  # eager once: one-time initialisation and the scratch pool's first allocation happen here
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        step()
+    g = gen(78)
+    for replay in range(3):
+        # new inputs in place (the graph holds the addresses), eager work and a synchronisation between the replays
+        w["q"].copy_((torch.randn(w["q"].shape, generator=g) * 0.25).half())
+        w["new_k"].copy_((torch.randn(w["new_k"].shape, generator=g) * 0.25).half())
+        w["new_v"].copy_((torch.randn(w["new_v"].shape, generator=g) * 0.25).half())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got_logits, got_out = logits.clone(), out.clone()
+        logits.zero_()
+        out.zero_()
+        with torch.cuda.stream(stream):
+            step()
+        stream.synchronize()
+        assert_bit_equal(got_logits, logits, f"replay {replay}: score rows")
+        assert_bit_equal(got_out, out, f"replay {replay}: decode output")
+        ref = torch.zeros(w["q"].shape, dtype=torch.float64)
+        O.token_softmax_reducev(logits.cpu(), w["v_cache"].cpu(), ref, w["b_loc"].cpu(), w["b_start_loc"].cpu(), w["b_seq_len"].cpu(), mil, 0, exact=True)
+        assert_close(got_out, ref, what=f"replay {replay}: decode output vs float64", **TOL[torch.float16])
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
