@@ -3,10 +3,13 @@
  *
  * This header carries the part of the DIOPI C ABI that the operator library
  * and its caller share: value types, opaque handles and the callbacks the
- * library imports from whoever owns the tensors.  Every declaration below is
- * binary- and source-compatible with the reference header it restates
- * (reference: proto/include/diopi/diopirt.h, line numbers cited per block), so
- * a translation unit may be compiled against either header directory.
+ * library imports from whoever owns the tensors.  Only what the LLaMA inference
+ * operators touch is restated; every declaration that is here is binary- and
+ * source-compatible with the reference header (reference:
+ * proto/include/diopi/diopirt.h, line numbers cited per block), so the
+ * operators' translation units compile against either header directory.  The
+ * scalar, memory-format, reduction and rounding-mode types of the reference
+ * header (diopirt.h:81-96) have no user on this path and are left out.
  *
  * Direction of the calls:
  *   caller  --diopiXxx(ctx, tensors...)-->  operator library (functions_ext.h)
@@ -29,11 +32,10 @@
 extern "C" {
 #endif
 
-/* reference: diopirt.h:22-25 */
+/* interface version this library reports (reference: diopirt.h:22-24) */
 #define DIOPI_VER_MAJOR 1
 #define DIOPI_VER_MINOR 0
 #define DIOPI_VER_PATCH 0
-#define DIOPI_VERSION (DIOPI_VER_MAJOR * 1000 + DIOPI_VER_MINOR * 100 + DIOPI_VER_PATCH)
 
 /* A borrowed array of int64 (shapes, strides, normalized_shape).  Passed by
  * value; the pointee stays owned by whoever produced it.  reference: diopirt.h:27-30 */
@@ -70,20 +72,6 @@ typedef enum {
     diopi_dtype_unsupported = 255
 } diopiDtype_t;
 
-/* reference: diopirt.h:81-87 */
-typedef struct {
-    diopiDtype_t stype;
-    union {
-        double fval;
-        int64_t ival;
-    };
-} diopiScalar_t;
-
-/* reference: diopirt.h:89-93 (unused by the LLaMA inference operators, kept for layout parity) */
-typedef enum { Contiguous = 0, ChannelsLast = 1, ChannelsLast3d = 2, Preserve = 3, ChannelsLast1d = 4 } diopiMemoryFormat_t;
-typedef enum { ReductionNone, ReductionMean, ReductionSum, ReductionEND } diopiReduction_t;
-typedef enum { RoundModeNone, RoundModeTrunc, RoundModeFloor, RoundModeEND } diopiRoundMode_t;
-
 /* Opaque handles: the library only ever passes them back to the callbacks.
  * reference: diopirt.h:98-112 */
 struct diopiContext;
@@ -97,40 +85,36 @@ typedef const struct diopiGenerator* diopiConstGeneratorHandle_t;
 /* The native stream of the device runtime; here a hipStream_t. */
 typedef void* diopiStreamHandle_t;
 
-/* reference: diopirt.h:117 */
-extern DIOPI_API const char* diopiGetVersion();
-
 /* ---- tensor accessors, implemented by the caller (reference: diopirt.h:122-140) ----
- * diopiGetTensorData already includes any storage offset. Shape/Stride return
- * pointers into caller-owned memory that lives as long as the tensor. */
-extern DIOPI_RT_API diopiError_t diopiGetTensorData(diopiTensorHandle_t th, void**);
-extern DIOPI_RT_API diopiError_t diopiGetTensorDataConst(diopiConstTensorHandle_t th, const void**);
-extern DIOPI_RT_API diopiError_t diopiGetTensorShape(diopiConstTensorHandle_t th, diopiSize_t* size);
-extern DIOPI_RT_API diopiError_t diopiGetTensorStride(diopiConstTensorHandle_t th, diopiSize_t* stride);
-extern DIOPI_RT_API diopiError_t diopiGetTensorDtype(diopiConstTensorHandle_t th, diopiDtype_t* dtype);
-extern DIOPI_RT_API diopiError_t diopiGetTensorNumel(diopiConstTensorHandle_t th, int64_t* numel);
-/* the following accessors are optional on the caller's side: test for null before use */
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorDevice(diopiConstTensorHandle_t th, diopiDevice_t* device);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorElemSize(diopiConstTensorHandle_t th, int64_t* itemsize);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStoragePtr(diopiConstTensorHandle_t th, void** pStoragePtr);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStorageOffset(diopiConstTensorHandle_t th, int64_t* pOffset);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStorageNbytes(diopiConstTensorHandle_t th, size_t* pNbytes);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetTensorDeviceIndex(diopiConstTensorHandle_t th, diopiDeviceIndex_t* pDevIndex);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiGetCurrentDeviceIndex(diopiDeviceIndex_t* pDevIndex);
+ * The data pointer already includes any storage offset.  Shape and stride come
+ * back as borrowed arrays that live as long as the tensor. */
+diopiError_t diopiGetTensorData(diopiTensorHandle_t tensor, void** data);
+diopiError_t diopiGetTensorDataConst(diopiConstTensorHandle_t tensor, const void** data);
+diopiError_t diopiGetTensorShape(diopiConstTensorHandle_t tensor, diopiSize_t* shape);
+diopiError_t diopiGetTensorStride(diopiConstTensorHandle_t tensor, diopiSize_t* strideInElements);
+diopiError_t diopiGetTensorDtype(diopiConstTensorHandle_t tensor, diopiDtype_t* dtype);
+diopiError_t diopiGetTensorNumel(diopiConstTensorHandle_t tensor, int64_t* count);
+/* Optional on the caller's side (weak): test the address before calling. */
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorDevice(diopiConstTensorHandle_t tensor, diopiDevice_t* where);
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorElemSize(diopiConstTensorHandle_t tensor, int64_t* bytesPerElement);
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStoragePtr(diopiConstTensorHandle_t tensor, void** storage);
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStorageOffset(diopiConstTensorHandle_t tensor, int64_t* offset);
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorStorageNbytes(diopiConstTensorHandle_t tensor, size_t* bytes);
+DIOPI_ATTR_WEAK diopiError_t diopiGetTensorDeviceIndex(diopiConstTensorHandle_t tensor, diopiDeviceIndex_t* index);
+DIOPI_ATTR_WEAK diopiError_t diopiGetCurrentDeviceIndex(diopiDeviceIndex_t* index);
 
 /* ---- stream and scratch memory, implemented by the caller (reference: diopirt.h:145-150) ----
- * Everything obtained through diopiRequireTensor/diopiRequireBuffer belongs to
- * the context: the library never frees it and never keeps the pointer past
- * the call that asked for it. */
-extern DIOPI_RT_API diopiError_t diopiGetStream(diopiContextHandle_t ctx, diopiStreamHandle_t* stream);
-extern DIOPI_RT_API diopiError_t diopiRequireTensor(diopiContextHandle_t ctx, diopiTensorHandle_t* tensor, const diopiSize_t* size, const diopiSize_t* stride,
-                                                    const diopiDtype_t dtype, const diopiDevice_t device);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiRequireBuffer(diopiContextHandle_t ctx, diopiTensorHandle_t* tensor, int64_t num_bytes,
-                                                                    diopiDevice_t device);
+ * Whatever diopiRequireTensor / diopiRequireBuffer hand out belongs to the
+ * context: the library never frees it and never keeps the pointer past the
+ * call that asked for it.  A null stride asks for a dense tensor. */
+diopiError_t diopiGetStream(diopiContextHandle_t ctx, diopiStreamHandle_t* nativeStream);
+diopiError_t diopiRequireTensor(diopiContextHandle_t ctx, diopiTensorHandle_t* made, const diopiSize_t* shape, const diopiSize_t* strideOrNull,
+                                const diopiDtype_t dtype, const diopiDevice_t where);
+DIOPI_ATTR_WEAK diopiError_t diopiRequireBuffer(diopiContextHandle_t ctx, diopiTensorHandle_t* made, int64_t bytes, diopiDevice_t where);
 
 /* ---- profiler scopes, optional (reference: diopirt.h:161-162) ---- */
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiRecordStart(const char* record_name, void** record);
-extern DIOPI_RT_API DIOPI_ATTR_WEAK diopiError_t diopiRecordEnd(void** record);
+DIOPI_ATTR_WEAK diopiError_t diopiRecordStart(const char* scopeName, void** scope);
+DIOPI_ATTR_WEAK diopiError_t diopiRecordEnd(void** scope);
 
 #if defined(__cplusplus)
 }
