@@ -4,6 +4,7 @@
 // provides to an operator library: tensor accessors, the context's stream and
 // context-owned scratch tensors.  Scratch comes from a per-context pool so that
 // repeated operator calls do not hit hipMalloc/hipFree.
+#include <conform_test.h>
 #include <diopirt_hip.h>
 #include <hip/hip_runtime.h>
 
@@ -306,5 +307,74 @@ diopiError_t diopiRequireBuffer(diopiContextHandle_t ctx, diopiTensorHandle_t* t
 
 diopiError_t diopiRecordStart(const char*, void**) { return diopiSuccess; }
 diopiError_t diopiRecordEnd(void**) { return diopiSuccess; }
+
+// ---------------------------------------------------------------------------
+// The device hooks of conform_test.h, through which the reference's harness reaches the device
+// (CUDA versions: impl/torch/test/conform_test.cpp:27-83).
+// ---------------------------------------------------------------------------
+
+static diopiError_t hookStatus(hipError_t err, const char* what) {
+    if (err == hipSuccess) return diopiSuccess;
+    std::fprintf(stderr, "%s failed: %s\n", what, hipGetErrorString(err));
+    (void)hipGetLastError();
+    return diopiErrorOccurred;
+}
+
+void* device_malloc(uint64_t bytes) {
+    void* ptr = nullptr;
+    if (hookStatus(hipMalloc(&ptr, bytes > 0 ? bytes : 1), "device_malloc") != diopiSuccess) return nullptr;
+    return ptr;
+}
+
+void device_free(void* ptr) {
+    if (ptr != nullptr) (void)hookStatus(hipFree(ptr), "device_free");
+}
+
+diopiError_t device_make_stream(diopiStreamHandle_t* stream) {
+    if (stream == nullptr) return diopiErrorOccurred;
+    hipStream_t made = nullptr;
+    const diopiError_t status = hookStatus(hipStreamCreate(&made), "device_make_stream");
+    *stream = made;
+    return status;
+}
+
+diopiError_t device_destroy_stream(diopiStreamHandle_t stream) {
+    return hookStatus(hipStreamDestroy(static_cast<hipStream_t>(stream)), "device_destroy_stream");
+}
+
+diopiError_t device_synchronize_stream(diopiStreamHandle_t stream) {
+    return hookStatus(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "device_synchronize_stream");
+}
+
+diopiError_t device_memcpy_h2d_async(diopiStreamHandle_t stream, void* deviceDst, const void* hostSrc, uint64_t bytes) {
+    if (bytes == 0) return diopiSuccess;
+    return hookStatus(hipMemcpyAsync(deviceDst, hostSrc, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)), "device_memcpy_h2d_async");
+}
+
+diopiError_t device_memcpy_d2h_async(diopiStreamHandle_t stream, void* hostDst, const void* deviceSrc, uint64_t bytes) {
+    if (bytes == 0) return diopiSuccess;
+    return hookStatus(hipMemcpyAsync(hostDst, deviceSrc, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)), "device_memcpy_d2h_async");
+}
+
+diopiError_t device_memcpy_d2d_async(diopiStreamHandle_t stream, void* deviceDst, const void* deviceSrc, uint64_t bytes) {
+    if (bytes == 0) return diopiSuccess;
+    return hookStatus(hipMemcpyAsync(deviceDst, deviceSrc, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)), "device_memcpy_d2d_async");
+}
+
+diopiError_t initLibrary(void) { return diopiSuccess; }
+diopiError_t finalizeLibrary(void) { return diopiSuccess; }
+
+diopiError_t buildGeneratorState(diopiContextHandle_t ctx, diopiTensorHandle_t out) {
+    if (ctx == nullptr || out == nullptr) return diopiErrorOccurred;
+    const int64_t stateBytes = 808;
+    const diopiSize_t shape{&stateBytes, 1};
+    diopiTensorHandle_t state = nullptr;
+    const diopiError_t status = diopiRequireTensor(ctx, &state, &shape, nullptr, diopi_dtype_uint8, diopi_host);
+    if (status != diopiSuccess) return status;
+    std::memset(state->data, 0, static_cast<size_t>(stateBytes));
+    *out = *state;      // `out` now views the context's block, which stays in the context's hands
+    out->capacity = 0;
+    return diopiSuccess;
+}
 
 }  // extern "C"

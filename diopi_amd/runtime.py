@@ -129,6 +129,21 @@ class _Libs:
         rt.diopirtEventElapsedMs.restype = ctypes.c_float
         rt.diopirtItemsize.argtypes = [i32]
         rt.diopirtItemsize.restype = i64
+        # the device hooks of the reference's harness (conform_test.h:28-43)
+        u64 = ctypes.c_uint64
+        rt.device_malloc.restype, rt.device_malloc.argtypes = vp, [u64]
+        rt.device_free.restype, rt.device_free.argtypes = None, [vp]
+        for name in ("device_memcpy_h2d_async", "device_memcpy_d2h_async", "device_memcpy_d2d_async"):
+            getattr(rt, name).restype, getattr(rt, name).argtypes = i32, [vp, vp, vp, u64]
+        rt.device_make_stream.restype, rt.device_make_stream.argtypes = i32, [ctypes.POINTER(vp)]
+        rt.device_destroy_stream.restype, rt.device_destroy_stream.argtypes = i32, [vp]
+        rt.device_synchronize_stream.restype, rt.device_synchronize_stream.argtypes = i32, [vp]
+        rt.initLibrary.restype, rt.initLibrary.argtypes = i32, []
+        rt.finalizeLibrary.restype, rt.finalizeLibrary.argtypes = i32, []
+        rt.buildGeneratorState.restype, rt.buildGeneratorState.argtypes = i32, [vp, vp]
+        rt.diopiGetTensorNumel.restype, rt.diopiGetTensorNumel.argtypes = i32, [vp, ctypes.POINTER(i64)]
+        rt.diopiGetTensorDtype.restype, rt.diopiGetTensorDtype.argtypes = i32, [vp, ctypes.POINTER(i32)]
+        rt.diopiGetTensorDevice.restype, rt.diopiGetTensorDevice.argtypes = i32, [vp, ctypes.POINTER(i32)]
 
         for name in ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString"):
             getattr(impl, name).restype = ctypes.c_char_p

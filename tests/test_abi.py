@@ -141,3 +141,32 @@ def test_runtime_scratch_pool_on_host():
     rtl.diopiGetTensorData(h, ctypes.byref(p2))
     assert p1.value == p2.value and ctx.malloc_count == 1
     ctx.close()
+
+
+HOOKS = ["device_malloc", "device_free", "device_memcpy_h2d_async", "device_memcpy_d2h_async", "device_memcpy_d2d_async", "device_make_stream",
+         "device_destroy_stream", "device_synchronize_stream", "initLibrary", "finalizeLibrary", "buildGeneratorState"]
+REF_HOOKS_HEADER = "/root/reference/diopi_test/diopi_stub/include/conform_test.h"
+
+
+def test_runtime_defines_the_harness_hooks():
+    """The device hooks the reference's harness links against (conform_test.h:28-43) are declared in
+    include/conform_test.h and defined by the HIP runtime library."""
+    text = open(os.path.join(ROOT, "include", "conform_test.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(\w+)\s*\(", text)) - {"defined"}
+    assert declared == set(HOOKS)
+    rt_defined, _ = _nm(rt.RT_LIB_PATH)
+    assert set(HOOKS) <= rt_defined
+    # without a device the set-up hooks still answer
+    rtl = rt.libs().rt
+    assert rtl.initLibrary() == 0 and rtl.finalizeLibrary() == 0
+
+
+@pytest.mark.skipif(not os.path.isfile(REF_HOOKS_HEADER), reason="reference headers not present")
+def test_hook_declarations_agree_with_the_reference_header():
+    """Both headers in one translation unit: with C linkage a differing prototype is a compile error."""
+    own = os.path.join(ROOT, "include", "conform_test.h")
+    for first, second in ((REF_HOOKS_HEADER, own), (own, REF_HOOKS_HEADER)):
+        cmd = ["g++", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I", REF_INCLUDE, "-include", first, "-include", second, "/dev/null"]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr[-4000:]

@@ -1064,6 +1064,74 @@ def test_decode_step_in_a_hip_graph_replays_like_eager():
         assert_close(got_out, ref, what=f"replay {replay}: decode output vs float64", **TOL[torch.float16])
 
 
+# ----------------------------------------------------------------------------- the reference harness's device hooks
+def test_harness_hooks_drive_an_operator_without_torch_on_the_device():
+    """The way diopi_test reaches the device (conform_test.h:28-43; litert.cpp:370-376): memory from device_malloc,
+    copies and synchronisation on a stream from device_make_stream, the operator enqueued on that stream."""
+    import ctypes as C
+    rtl, impl = rt.libs().rt, rt.libs().impl
+    vp = C.c_void_p
+
+    assert rtl.initLibrary() == 0
+    stream = vp()
+    assert rtl.device_make_stream(C.byref(stream)) == 0 and stream.value
+
+    # byte round trip host -> device -> device -> host, odd size
+    rng = np.random.default_rng(5)
+    src = rng.integers(0, 256, size=1_000_003, dtype=np.uint8)
+    back = np.zeros_like(src)
+    a, b = rtl.device_malloc(src.nbytes), rtl.device_malloc(src.nbytes)
+    assert a and b
+    assert rtl.device_memcpy_h2d_async(stream, a, src.ctypes.data, src.nbytes) == 0
+    assert rtl.device_memcpy_d2d_async(stream, b, a, src.nbytes) == 0
+    assert rtl.device_memcpy_d2h_async(stream, back.ctypes.data, b, src.nbytes) == 0
+    assert rtl.device_synchronize_stream(stream) == 0
+    assert np.array_equal(src, back)
+    assert rtl.device_memcpy_d2d_async(stream, b, a, 0) == 0  # empty copies are legal
+    rtl.device_free(a)
+    rtl.device_free(b)
+
+    # RMSNorm at the reference's case shape (diopi_configs.py:9153), every buffer owned by the hooks
+    n1, n2, eps = 12, 32, 1e-6
+    x = rng.standard_normal((n1, n2)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, n2).astype(np.float32)
+    out, inv = np.zeros_like(x), np.zeros(n1, np.float32)
+    dx, dw, dout, dinv = (rtl.device_malloc(t.nbytes) for t in (x, w, out, inv))
+    assert rtl.device_memcpy_h2d_async(stream, dx, x.ctypes.data, x.nbytes) == 0
+    assert rtl.device_memcpy_h2d_async(stream, dw, w.ctypes.data, w.nbytes) == 0
+    ctx = rtl.diopirtContextCreate(stream)
+
+    def wrap(ptr, *shape):
+        dims = (C.c_int64 * len(shape))(*shape)
+        return rtl.diopirtTensorWrap(ptr, dims, None, len(shape), int(rt.Dtype.float32), int(rt.Device.AIChip))
+
+    tx, tw, tout, tinv = wrap(dx, n1, n2), wrap(dw, n2), wrap(dout, n1, n2), wrap(dinv, n1)
+    ret = impl.diopiRMSNorm(ctx, tout, tinv, tx, rt.Sizes([n2]).c, tw, None, eps)
+    assert ret == 0, rt.get_last_error_string()
+    assert rtl.device_memcpy_d2h_async(stream, out.ctypes.data, dout, out.nbytes) == 0
+    assert rtl.device_memcpy_d2h_async(stream, inv.ctypes.data, dinv, inv.nbytes) == 0
+    assert rtl.device_synchronize_stream(stream) == 0
+    want_out, want_inv = O.rms_norm(torch.from_numpy(x), (n2,), torch.from_numpy(w), None, eps)
+    assert_close(torch.from_numpy(out), want_out, what="RMSNorm through the harness hooks", **TOL[torch.float32])
+    assert_close(torch.from_numpy(inv), want_inv, what="inv_rms through the harness hooks", **TOL[torch.float32])
+
+    # the generator-state hook hands out 808 host bytes owned by the context
+    state = rtl.diopirtTensorWrap(None, (C.c_int64 * 1)(0), None, 1, int(rt.Dtype.uint8), int(rt.Device.Host))
+    assert rtl.buildGeneratorState(ctx, state) == 0
+    numel, dtype, where = C.c_int64(), C.c_int(), C.c_int()
+    assert rtl.diopiGetTensorNumel(state, C.byref(numel)) == 0 and numel.value == 808
+    assert rtl.diopiGetTensorDtype(state, C.byref(dtype)) == 0 and dtype.value == int(rt.Dtype.uint8)
+    assert rtl.diopiGetTensorDevice(state, C.byref(where)) == 0 and where.value == int(rt.Device.Host)
+
+    for t in (tx, tw, tout, tinv, state):
+        rtl.diopirtTensorDestroy(t)
+    rtl.diopirtContextDestroy(ctx)
+    for ptr in (dx, dw, dout, dinv):
+        rtl.device_free(ptr)
+    assert rtl.device_destroy_stream(stream) == 0
+    assert rtl.finalizeLibrary() == 0
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
