@@ -184,7 +184,10 @@ def main():
             # full-width tables for the fused in-place operator (same angles in both halves)
             s["cos2"] = torch.cat((s["cos"], s["cos"]), -1).contiguous()
             s["sin2"] = torch.cat((s["sin"], s["sin"]), -1).contiguous()
-            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "out", "inv", "q", "k", "cos", "sin", "qo", "ko", "cos2", "sin2")})
+            # hidden state and residual of the fused in-place normalisation (they keep accumulating: same work every step)
+            s["hid"] = s["x"].clone()
+            s["res"] = torch.zeros_like(s["x"])
+            hs.append({k: Tensor(s[k]) for k in ("x", "weight", "out", "inv", "q", "k", "cos", "sin", "qo", "ko", "cos2", "sin2", "hid", "res")})
 
         def norm(i):
             h = hs[i % 3]
@@ -200,9 +203,15 @@ def main():
             h = hs[i % 3]
             check(impl.diopiRotaryEmbeddingV2(ctx.handle, h["qo"].handle, h["ko"].handle, h["cos2"].handle, h["sin2"].handle, D), "diopiRotaryEmbeddingV2")
 
+        def addnorm(i):
+            h = hs[i % 3]
+            check(impl.diopiFusedAddRootMeanSquareNormInp(ctx.handle, h["hid"].handle, h["res"].handle, None, h["weight"].handle, 1e-6),
+                  "diopiFusedAddRootMeanSquareNormInp")
+
         ms_n = timed(norm)
         ms_r = timed(rot)
         ms_r2 = timed(rot2)
+        ms_an = timed(addnorm)
         cpu_n = cpu_r = None
         if not args.no_cpu:
             xc, wc = sets[0]["x"].cpu(), sets[0]["weight"].cpu()
@@ -215,6 +224,8 @@ def main():
         record("diopiRotaryEmbedding x2 (q,k)", "cfg2 bf16 [16384,32,128]", ms_r, 2 * W.rotary_bytes(T, H, D, 2), "hbm", "bf16", cpu_r)
         record("diopiRotaryEmbeddingV2 (q,k in place, one launch)", "cfg2 bf16 [16384,32,128] x2", ms_r2, 2 * 2 * T * H * D * 2 + 2 * T * D * 2, "hbm", "bf16",
                None, note="widening beyond the seven hot-path operators; bytes = read+write of q and k, full-width cos/sin once")
+        record("diopiFusedAddRootMeanSquareNormInp (residual add + RMSNorm, in place)", "cfg2 bf16 [16384,4096] x2", ms_an, 4 * T * n2 * 2 + n2 * 2, "hbm",
+               "bf16", None, note="widening beyond the seven hot-path operators; bytes = read+write of the hidden state and of the residual, scale once")
         del sets, hs
         torch.cuda.empty_cache()
 

@@ -138,6 +138,27 @@ def rms_norm_backward(grad_outputs: Sequence[torch.Tensor], input: torch.Tensor,
     return out
 
 
+def root_mean_square_norm_inp(inoutput: torch.Tensor, scale: torch.Tensor, eps: float, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """In-place RMS normalisation of every row (functions_lmdeploy.h:31-38 of the reference)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, inoutput):
+        keep, h = _handles(inoutput, scale)
+        ret = rt.libs().impl.diopiRootMeanSquareNormInp(ctx.handle, h[0], h[1], float(eps))
+    check_returncode(ret, "diopiRootMeanSquareNormInp")
+    return inoutput
+
+
+def fused_add_root_mean_square_norm_inp(inoutput: torch.Tensor, residual: torch.Tensor, bias: Optional[torch.Tensor], scale: torch.Tensor, eps: float,
+                                        ctx: Optional[rt.Context] = None):
+    """residual += inoutput + bias; inoutput = RMSNorm(residual) * scale (functions_lmdeploy.h:40-49 of the reference)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, inoutput):
+        keep, h = _handles(inoutput, residual, bias, scale)
+        ret = rt.libs().impl.diopiFusedAddRootMeanSquareNormInp(ctx.handle, h[0], h[1], h[2], h[3], float(eps))
+    check_returncode(ret, "diopiFusedAddRootMeanSquareNormInp")
+    return inoutput, residual
+
+
 def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor, ctx: Optional[rt.Context] = None) -> torch.Tensor:
     ctx = _ctx(ctx)
     with _on_stream(ctx, out):

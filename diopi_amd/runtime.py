@@ -167,11 +167,13 @@ class _Libs:
         impl.diopiMultiHeadAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, dbl, ctypes.c_bool, ctypes.c_bool, dbl, vp, vp, vp, vp]
         impl.diopiPagedAttention.argtypes = [vp, vp, vp, vp, vp, vp, _SizeStruct, i64, i64, i64, vp, i64]
         impl.diopiPromptFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, _SizeStruct, i64, i64, i64, i64]
+        impl.diopiRootMeanSquareNormInp.argtypes = [vp, vp, vp, ctypes.c_float]
+        impl.diopiFusedAddRootMeanSquareNormInp.argtypes = [vp, vp, vp, vp, vp, ctypes.c_float]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
 
-# Every symbol include/diopi/functions.h and include/diopi/functions_ext.h declare.
+# Every symbol include/diopi/functions.h, functions_ext.h and functions_lmdeploy.h declare.
 OPERATOR_SYMBOLS = (
     "diopiRotaryEmbedding",
     "diopiRotaryEmbeddingV2",
@@ -189,6 +191,8 @@ OPERATOR_SYMBOLS = (
     "diopiMultiHeadAttentionVarLen",
     "diopiPagedAttention",
     "diopiPromptFlashAttention",
+    "diopiRootMeanSquareNormInp",
+    "diopiFusedAddRootMeanSquareNormInp",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

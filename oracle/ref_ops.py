@@ -1,5 +1,6 @@
 """CPU oracle for the LLaMA-inference operators (the seven of the hot path, diopiRotaryEmbeddingV2,
-diopiApplyPenalty/V2 and the flash / prompt / paged attention forms).  TEST INFRASTRUCTURE ONLY.
+diopiApplyPenalty/V2, the flash / prompt / paged attention forms and the two in-place RMS normalisations of
+the lmdeploy set).  TEST INFRASTRUCTURE ONLY.
 
 This module restates, on the CPU with plain ATen (torch) and numpy calls, what the reference
 computes for each operator.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
@@ -12,6 +13,9 @@ rms_norm                     impl/torch/functions/functions_ext.cpp:66-80,
                              functions_ext/layer_norm_cuda_kernel.cu:321-366 (cuApplyRMSNorm),
                              functions_ext/rmsnorm.cu:17-28; Python twin customized_test.py:392-403
 rms_norm_backward            functions_ext.cpp:82-107, layer_norm_cuda_kernel.cu:402, 444, 572-717
+root_mean_square_norm_inp    proto/include/diopi/functions_lmdeploy.h:31-38 (declaration and one sentence only:
+fused_add_root_mean_         the reference tree has no implementation, Python statement or test case of the
+  square_norm_inp            lmdeploy operators), 40-49: "1.(res + inout + bias) = new_res 2.RMSNorm(new_res) = inout"
 rotary_emb                   functions_ext.cpp:43-64, functions_ext/rotary.cu:26-44;
                              customized_test.py:374-390
 rotary_emb_v2                customized_test.py:843-852 (the torch implementation has no body for
@@ -43,10 +47,18 @@ Grouped-query attention (H = G * Hkv query heads over Hkv cache heads) is an ext
 decode operators: query head h reads cache head h // G (the grouping rule of the reference's
 flash-attention test, customized_test.py:466-472).  With G == 1 the functions are the reference's.
 
-How each function is pinned (see tests/test_oracle.py; none is "parity unpinned"):
+How each function is pinned (see tests/test_oracle.py).  None of the reference's own statements is "parity
+unpinned".  For the two lmdeploy normalisations the header's sentence is all the reference holds: the value
+is pinned to that sentence by the checks below; WHERE the 16-bit roundings fall is taken from lmdeploy's
+published turbomind kernels (llama_kernels.cu; the reference records no version of them) and is "parity
+unpinned" - the candidate orders differ by at most one unit in the last place of the element type, well
+inside the 1e-2 bar of 16-bit tensors, and not at all in fp32 beyond 1e-6:
   rms_norm / backward  closed forms (constant rows, +-1 rows, scale invariance, sum((out/w)^2)),
                        float64 autograd of the textbook formula, the identity
                        sum_l x_l*grad_input_l = eps*inv_rms^3*sum_l g_l*x_l, column sums in float64
+  root_mean_square_norm_inp / fused_add_...  with a zero residual and no bias both are rms_norm (pinned
+                       above) on the same rows; the new residual is the float64 sum of its three terms; constant
+                       rows in closed form; sum((out/scale)^2) = n*ms/(ms+eps); fused = add, then the plain form
   rotary_emb           position 0 is the identity bit for bit, norm preservation per pair,
                        conj undoes the rotation, the reference's broadcasting shapes
                        (diopi_configs.py:9066-9074), empty tensors (9093)
@@ -144,6 +156,44 @@ def rms_norm_backward(grad_output: torch.Tensor, input: torch.Tensor, weight: to
         return grad_input.reshape(input.shape), grad_weight.reshape(weight.shape), (grad_bias.reshape(weight.shape) if with_bias else None)
     return (grad_input.to(input.dtype).reshape(input.shape), grad_weight.to(weight.dtype).reshape(weight.shape),
             grad_bias.to(weight.dtype).reshape(weight.shape) if with_bias else None)
+
+
+def root_mean_square_norm_inp(inoutput: torch.Tensor, scale: torch.Tensor, eps: float, exact: bool = False) -> torch.Tensor:
+    """functions_lmdeploy.h:31-38: every row times rsqrt(mean(row^2) + eps) times scale.  Returns the new inoutput.
+
+    Roundings (turbomind's rootMeanSquareNorm): fp32 sums, the normalised value rounded to the dtype, then its
+    product with scale rounded again - the same form as rms_norm above."""
+    n = inoutput.shape[-1]
+    if exact:
+        x = inoutput.double()
+        inv = 1.0 / torch.sqrt((x * x).sum(-1, keepdim=True) / n + eps)
+        return x * inv * scale.double()
+    x = inoutput.float()
+    inv = torch.rsqrt((x * x).sum(-1, keepdim=True) / n + torch.tensor(eps, dtype=torch.float32))
+    normed = (x * inv).to(inoutput.dtype)
+    return (normed.float() * scale.float()).to(inoutput.dtype)
+
+
+def fused_add_root_mean_square_norm_inp(inoutput: torch.Tensor, residual: torch.Tensor, bias: Optional[torch.Tensor], scale: torch.Tensor,
+                                        eps: float, exact: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """functions_lmdeploy.h:40-49: new_res = res + inout + bias, inout = RMSNorm(new_res) * scale.
+    Returns (new inoutput, new residual).
+
+    Roundings (turbomind's fusedAddBiasResidualNorm): the three-term sum is formed in fp32, its squares are
+    summed unrounded, the stored residual is the sum rounded once, and the output is one rounding of
+    stored_residual * (inv * scale)."""
+    n = inoutput.shape[-1]
+    acc = torch.float64 if exact else torch.float32
+    s = residual.to(acc) + inoutput.to(acc)
+    if bias is not None:
+        s = s + bias.to(acc)
+    if exact:
+        inv = 1.0 / torch.sqrt((s * s).sum(-1, keepdim=True) / n + eps)
+        return s * inv * scale.double(), s
+    inv = torch.rsqrt((s * s).sum(-1, keepdim=True) / n + torch.tensor(eps, dtype=torch.float32))
+    stored = s.to(inoutput.dtype)
+    out = (stored.float() * (inv * scale.float())).to(inoutput.dtype)
+    return out, stored
 
 
 def rotary_emb(input: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, conj: bool, interleaved: bool = False, exact: bool = False) -> torch.Tensor:

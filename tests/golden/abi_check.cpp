@@ -6,13 +6,18 @@
 #include <diopi/diopirt.h>
 #include <diopi/functions.h>
 #include <diopi/functions_ext.h>
+#include <diopi/functions_lmdeploy.h>
 #else
 #include <diopi/diopirt.h>
 #include <diopi/functions.h>
 #include <diopi/functions_ext.h>
+#include <diopi/functions_lmdeploy.h>
 #endif
 
 extern "C" {
+diopiError_t diopiRootMeanSquareNormInp(diopiContextHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t, float);
+diopiError_t diopiFusedAddRootMeanSquareNormInp(diopiContextHandle_t, diopiTensorHandle_t, diopiTensorHandle_t, diopiConstTensorHandle_t,
+                                                diopiConstTensorHandle_t, float);
 const char* diopiGetVendorName();
 const char* diopiGetImplVersion();
 const char* diopiGetLastErrorString();

@@ -37,7 +37,7 @@ def _declared(header):
 
 def test_exports_match_headers():
     defined, undefined = _nm(rt.IMPL_LIB_PATH)
-    declared = _declared("functions_ext.h") | _declared("functions.h")
+    declared = _declared("functions_ext.h") | _declared("functions.h") | _declared("functions_lmdeploy.h")
     assert declared == set(rt.OPERATOR_SYMBOLS) | set(rt.INFO_SYMBOLS)
     exported = {s for s in defined if s.startswith("diopi")}
     assert exported == declared, f"exported {sorted(exported)} vs declared {sorted(declared)}"

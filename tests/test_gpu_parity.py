@@ -211,6 +211,90 @@ def test_rms_norm_config2_full_size():
     assert_close(o16, r16, rtol=1e-2, atol=1e-2, what="fp32 -> bf16 rms_norm")
 
 
+# ----------------------------------------------------------------------------- in-place RMS normalisations (lmdeploy set)
+def _inplace_norm_case(shape, dt, with_bias, seed, eps=1e-6, offset=0):
+    g = gen(seed)
+    n = shape[-1]
+
+    def dense(*sh):
+        # offset > 0: a dense view whose first element is not 16-byte aligned
+        flat = torch.randn(int(np.prod(sh)) + offset, generator=g).to(dt).to(DEV)
+        return flat[offset:].view(*sh)
+
+    x, r = dense(*shape), dense(*shape)
+    b = dense(n) if with_bias else None
+    w = (dense(n).abs() + 0.5).to(dt)
+    xc, rc, bc, wc = x.cpu(), r.cpu(), (None if b is None else b.cpu()), w.cpu()
+    before = snapshot(b, w)
+    # plain form on a copy of x
+    y = x.clone() if offset == 0 else dense(*shape).copy_(x)
+    F.root_mean_square_norm_inp(y, w, eps)
+    assert_close(y, O.root_mean_square_norm_inp(xc, wc, eps), what=f"plain {shape} {dt}", **TOL[dt])
+    assert_close(y, O.root_mean_square_norm_inp(xc, wc, eps, exact=True), what=f"plain {shape} {dt} vs float64", **TOL[dt])
+    # fused form
+    F.fused_add_root_mean_square_norm_inp(x, r, b, w, eps)
+    want_out, want_res = O.fused_add_root_mean_square_norm_inp(xc, rc, bc, wc, eps)
+    e_out, e_res = O.fused_add_root_mean_square_norm_inp(xc, rc, bc, wc, eps, exact=True)
+    if dt == torch.float32:
+        assert_close(r, want_res, rtol=0, atol=0, what=f"fused {shape} {dt}: residual (fp32 sum, same order)")
+    else:
+        assert_bit_equal(r, want_res, f"fused {shape} {dt}: residual is the sum rounded once")
+    assert_close(x, want_out, what=f"fused {shape} {dt} bias={with_bias}", **TOL[dt])
+    assert_close(x, e_out, what=f"fused {shape} {dt} vs float64", **TOL[dt])
+    assert_close(r, e_res, what=f"fused residual {shape} {dt} vs float64", **TOL[dt])
+    assert_unmodified(before, b, w)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "bfloat16"])
+def test_inplace_norms_shapes(dtype):
+    dt = TORCH_DTYPES[dtype]
+    # the reference's rms_norm case shape, the model widths, rows with a tail, rows that are no packet multiple,
+    # rows longer than the register form holds, a 3-d input, unaligned views
+    for i, shape in enumerate([(12, 32), (7, 4096), (33, 8192), (5, 100), (3, 4104), (4, 11008), (2, 40000), (2, 3, 256), (1, 8)]):
+        for with_bias in (False, True):
+            say("in-place norm", shape, dtype, with_bias)
+            _inplace_norm_case(shape, dt, with_bias, 500 + i)
+    for shape in [(9, 4096), (4, 512)]:
+        say("in-place norm, unaligned", shape, dtype)
+        _inplace_norm_case(shape, dt, True, 520, offset=1)
+
+
+def test_inplace_norms_full_size_and_against_the_separate_operators():
+    w = W.cfg2(DEV, seed=2)  # bf16 [16384, 4096]
+    x, wt, eps = w["x"], w["weight"], w["eps"]
+    g = gen(530)
+    res = torch.randn(x.shape, generator=g).to(x.dtype).to(DEV)
+    x0, r0 = x.clone(), res.clone()
+    F.fused_add_root_mean_square_norm_inp(x, res, None, wt, eps)
+    want_out, want_res = O.fused_add_root_mean_square_norm_inp(x0.cpu(), r0.cpu(), None, wt.cpu(), eps)
+    assert_bit_equal(res, want_res, "full size: residual")
+    assert_close(x, want_out, what="full size: fused output", **TOL[torch.bfloat16])
+    # the same step from the separate operators: an addition, then diopiRMSNorm on the stored sum
+    two_step = F.rms_norm(want_res.to(DEV), w["normalized_shape"], wt, None, eps)
+    assert_close(x, two_step, what="fused vs addition + diopiRMSNorm", **TOL[torch.bfloat16])
+    # the plain form is diopiRMSNorm in place: same roundings, so the same bits
+    y = x0.clone()
+    F.root_mean_square_norm_inp(y, wt, eps)
+    assert_bit_equal(y, F.rms_norm(x0, w["normalized_shape"], wt, None, eps), "plain form vs diopiRMSNorm")
+
+
+def test_inplace_norms_empty_and_argument_errors():
+    wt = torch.ones(64, device=DEV)
+    x = torch.zeros(0, 64, device=DEV)
+    F.root_mean_square_norm_inp(x, wt, 1e-6)
+    F.fused_add_root_mean_square_norm_inp(x, torch.zeros(0, 64, device=DEV), None, wt, 1e-6)
+    x = torch.randn(4, 64, device=DEV)
+    with pytest.raises(rt.DiopiException):
+        F.fused_add_root_mean_square_norm_inp(x, x, None, wt, 1e-6)  # one tensor in both roles
+    with pytest.raises(rt.DiopiException):
+        F.fused_add_root_mean_square_norm_inp(x, torch.randn(4, 32, device=DEV), None, wt, 1e-6)
+    with pytest.raises(rt.DiopiException):
+        F.root_mean_square_norm_inp(x, wt.half(), 1e-6)
+    with pytest.raises(rt.DiopiException):
+        F.root_mean_square_norm_inp(x.double(), wt.double(), 1e-6)
+    torch.cuda.synchronize()
+
+
 # ----------------------------------------------------------------------------- Rotary
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32", "float64"])
 def test_rotary_reference_cases(golden, dtype):

@@ -70,6 +70,68 @@ def test_rms_norm_modes_agree_and_match_python_twin(dtype):
     assert inv.dtype == torch.float32 and out.dtype == dtype
 
 
+# ----------------------------------------------------------------------------- in-place RMS normalisations (lmdeploy set)
+def test_inplace_norms_reduce_to_rms_norm_and_to_each_other():
+    g = rng(40)
+    x = torch.randn(6, 48, generator=g, dtype=torch.float64)
+    r = torch.randn(6, 48, generator=g, dtype=torch.float64)
+    b = torch.randn(48, generator=g, dtype=torch.float64)
+    w = torch.rand(48, generator=g, dtype=torch.float64) + 0.5
+    eps = 1e-5
+    want, _ = O.rms_norm(x, (48,), w, None, eps, exact=True)  # pinned by the tests above
+    assert_close(O.root_mean_square_norm_inp(x, w, eps, exact=True), want, 1e-13, 0, "plain form vs rms_norm")
+    out, res = O.fused_add_root_mean_square_norm_inp(x, torch.zeros_like(x), None, w, eps, exact=True)
+    assert_close(out, want, 1e-13, 0, "zero residual, no bias vs rms_norm")
+    assert_bit_equal(res, x, "zero residual, no bias: the new residual is the input")
+    # the new residual is the sum of its three terms, and the output is the plain form applied to it
+    out, res = O.fused_add_root_mean_square_norm_inp(x, r, b, w, eps, exact=True)
+    assert_close(res, x + r + b, 1e-14, 0, "new residual")
+    assert_close(out, O.root_mean_square_norm_inp(x + r + b, w, eps, exact=True), 1e-13, 0, "fused = add, then normalise")
+    # a dropped bias or residual term must show
+    assert (out - O.fused_add_root_mean_square_norm_inp(x, r, None, w, eps, exact=True)[0]).abs().max() > 1e-3
+    assert (out - O.fused_add_root_mean_square_norm_inp(x, torch.zeros_like(r), b, w, eps, exact=True)[0]).abs().max() > 1e-3
+
+
+def test_inplace_norms_closed_forms():
+    # constant rows: s = cr + cx + cb, out = scale * s / sqrt(s^2 + eps)
+    cx, cr, cb, eps = 1.5, -0.25, 2.0, 1e-2
+    n = 32
+    w = torch.linspace(0.5, 1.5, n, dtype=torch.float64)
+    x = torch.full((3, n), cx, dtype=torch.float64)
+    r = torch.full((3, n), cr, dtype=torch.float64)
+    b = torch.full((n,), cb, dtype=torch.float64)
+    s = cx + cr + cb
+    out, res = O.fused_add_root_mean_square_norm_inp(x, r, b, w, eps, exact=True)
+    assert_close(res, torch.full((3, n), s, dtype=torch.float64), 1e-15, 0, "constant rows: residual")
+    assert_close(out, (w * s / math.sqrt(s * s + eps)).expand(3, n), 1e-14, 0, "constant rows: output")
+    # energy identity: sum((out/scale)^2) = n * ms / (ms + eps)
+    g = rng(41)
+    y = torch.randn(5, 64, generator=g, dtype=torch.float64) * 3
+    w = torch.rand(64, generator=g, dtype=torch.float64) + 0.5
+    o = O.root_mean_square_norm_inp(y, w, eps, exact=True)
+    ms = (y * y).mean(-1)
+    assert_close(((o / w) ** 2).sum(-1), 64 * ms / (ms + eps), 1e-12, 0, "energy identity")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_inplace_norms_dtype_mode_is_close_to_exact_and_stores_a_rounded_residual(dtype):
+    g = rng(42)
+    x = torch.randn(9, 256, generator=g).to(dtype)
+    r = torch.randn(9, 256, generator=g).to(dtype)
+    b = torch.randn(256, generator=g).to(dtype)
+    w = (torch.rand(256, generator=g) + 0.5).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    out, res = O.fused_add_root_mean_square_norm_inp(x, r, b, w, 1e-6)
+    eo, er = O.fused_add_root_mean_square_norm_inp(x, r, b, w, 1e-6, exact=True)
+    assert out.dtype == dtype and res.dtype == dtype
+    if dtype == torch.float32:
+        assert_close(res, er, 2e-7, 1e-6, "the stored residual is the fp32 sum")  # absolute: the terms cancel
+    else:  # sums of three 16-bit values are exact in fp32 here, so one rounding is left
+        assert_bit_equal(res, er.to(dtype), "the stored residual is the exact sum rounded once")
+    assert_close(out, eo, tol, tol, "fused, dtype mode vs float64")
+    assert_close(O.root_mean_square_norm_inp(x, w, 1e-6), O.root_mean_square_norm_inp(x, w, 1e-6, exact=True), tol, tol, "plain, dtype mode vs float64")
+
+
 def test_rms_norm_backward_matches_float64_autograd():
     g = rng(3)
     for shape, ns in [((5, 5), (5,)), ((16, 64, 64), (64, 64)), ((3, 2, 16, 7, 8), (7, 8))]:
