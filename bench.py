@@ -75,6 +75,10 @@ def main():
     def check(ret, what):
         rt.check_returncode(ret, what)
 
+    class Timing(float):
+        """Average milliseconds per step of one timed region, with the median and minimum over its blocks."""
+        median = minimum = None
+
     def timed(step_fn, steps=K, warmup=Wm):
         """Average milliseconds per call of step_fn(i), events on the context's stream."""
         for i in range(warmup):
@@ -90,15 +94,23 @@ def main():
                 i += 1
             ctx.synchronize()
         torch.cuda.synchronize()
-        e0, e1 = rt.Event(), rt.Event()
-        e0.record(ctx)
-        for i in range(steps):
-            step_fn(i)
-        e1.record(ctx)
-        ms = e0.elapsed_ms(e1)
+        # one event before the K steps, one after each block of about a tenth of them: the K steps are timed as one
+        # region (the average), and the blocks give a median and a minimum without an event behind every launch
+        nblocks = max(1, min(10, steps // 5))
+        bounds = [round(b * steps / nblocks) for b in range(nblocks + 1)]
+        events = [rt.Event() for _ in range(nblocks + 1)]
+        events[0].record(ctx)
+        for b in range(nblocks):
+            for i in range(bounds[b], bounds[b + 1]):
+                step_fn(i)
+            events[b + 1].record(ctx)
+        ms = events[0].elapsed_ms(events[-1])
+        per_block = sorted(events[b].elapsed_ms(events[b + 1]) / (bounds[b + 1] - bounds[b]) for b in range(nblocks))
         ctx.synchronize()
         torch.cuda.synchronize()
-        return ms / steps
+        t = Timing(ms / steps)
+        t.median, t.minimum = per_block[len(per_block) // 2], per_block[0]
+        return t
 
     def cpu_time(fn, budget_s=3.0, min_reps=1, max_reps=5):
         """Median seconds of fn() on the host after one warm-up, bounded by a time budget."""
@@ -116,6 +128,8 @@ def main():
 
     def record(name, cfg, ms, work, bound, dtype, cpu=None, note=None):
         e = dict(op=name, config=cfg, dtype=dtype, ms=round(ms, 5), bound=bound)
+        if getattr(ms, "median", None) is not None:
+            e.update(ms_median=round(ms.median, 5), ms_min=round(ms.minimum, 5))
         if bound == "hbm":
             ach = work / (ms * 1e-3) / 1e9
             e.update(bytes=int(work), achieved_GBs=round(ach, 1), frac=round(ach / HBM_PEAK_GBS, 4))
