@@ -119,6 +119,24 @@ int diopirtDeviceCount(void) {
     return n;
 }
 
+int diopirtDeviceClockKHz(int device) {
+    int khz = 0;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, device) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return khz;
+}
+
+int diopirtDeviceComputeUnits(int device) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
 diopiContextHandle_t diopirtContextCreate(void* stream) {
     auto* ctx = new diopiContext();
     if (stream != nullptr) {

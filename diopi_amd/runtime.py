@@ -109,6 +109,8 @@ class _Libs:
         rt, impl = self.rt, self.impl
         vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
         rt.diopirtDeviceCount.restype = i32
+        rt.diopirtDeviceClockKHz.restype, rt.diopirtDeviceClockKHz.argtypes = i32, [i32]
+        rt.diopirtDeviceComputeUnits.restype, rt.diopirtDeviceComputeUnits.argtypes = i32, [i32]
         rt.diopirtContextCreate.restype = vp
         rt.diopirtContextCreate.argtypes = [vp]
         rt.diopirtContextDestroy.argtypes = [vp]

@@ -29,6 +29,10 @@ extern "C" {
 /* Number of HIP devices visible to the process (0 when there is none; never fails). */
 int diopirtDeviceCount(void);
 
+/* Maximum shader clock in kHz and number of compute units of a device (0 when the query fails). */
+int diopirtDeviceClockKHz(int device);
+int diopirtDeviceComputeUnits(int device);
+
 /* Create a context.  `stream` is an existing hipStream_t to adopt, or NULL to
  * let the context create its own non-blocking stream on first use. */
 diopiContextHandle_t diopirtContextCreate(void* stream);
