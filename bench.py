@@ -71,6 +71,15 @@ def main():
     K, Wm = args.steps, args.warmup
     only = set(x for x in args.only.split(",") if x)
     cores = torch.get_num_threads()
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    cpu_model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
 
     def check(ret, what):
         rt.check_returncode(ret, what)
@@ -447,6 +456,7 @@ def main():
         "config": {"workload": "cfg3 decode step fp16: 2x DestIndexCopyKV [64,32,128] -> cache [131072,32,128], TokenAttention + "
                                "TokenSoftmaxReduceV, batch 64, 32 heads x 128, b_loc [64,2048], seq_len ~U(512,2048)"},
         "roofline": None, "cpu_baseline": None, "ops": ops,
+        "host": {"cpu_model": cpu_model, "threads_used": cores},
         "peaks": {"hbm_GBs": HBM_PEAK_GBS, "mfma_f16_TFLOPs": MFMA_PEAK_TFLOPS, "device": device_peak},
     }
     if head is not None:
@@ -464,7 +474,8 @@ def main():
                             "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}
         if head["cpu"] is not None:
             c = head["cpu"]
-            line["cpu_baseline"] = {"value": c["tokens_per_s"], "unit": "tokens/s", "cores": c["cores"], "kind": "port", "sample": c["sample"]}
+            line["cpu_baseline"] = {"value": c["tokens_per_s"], "unit": "tokens/s", "cores": c["cores"], "kind": "port", "sample": c["sample"],
+                                    "cpu_model": cpu_model}
     print(json.dumps(line), flush=True)
 
 
