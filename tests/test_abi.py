@@ -170,3 +170,15 @@ def test_hook_declarations_agree_with_the_reference_header():
         cmd = ["g++", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I", REF_INCLUDE, "-include", first, "-include", second, "/dev/null"]
         res = subprocess.run(cmd, capture_output=True, text=True)
         assert res.returncode == 0, res.stderr[-4000:]
+
+
+C_CLIENT = os.path.join(os.path.dirname(rt.IMPL_LIB_PATH), "diopi_c_client")
+
+
+def test_c_host_links_and_loads():
+    """tests/golden/c_client.c, a host in plain C built by the package's Makefile against the public headers and
+    the two libraries: here (no device) it must link, load and read the library's identity."""
+    assert os.path.isfile(C_CLIENT), "run `python -c 'import __graft_entry__ as g; g.build()'` first"
+    res = subprocess.run([C_CLIENT], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "Device" in res.stdout.splitlines()[0] and res.stdout.strip().endswith("c client ok")

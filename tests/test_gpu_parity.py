@@ -1216,6 +1216,19 @@ def test_harness_hooks_drive_an_operator_without_torch_on_the_device():
     assert rtl.finalizeLibrary() == 0
 
 
+def test_c_host_runs_operators_through_the_c_abi():
+    """The plain-C host of tests/golden/c_client.c: RMSNorm against a double-precision loop and DestIndexCopyKV against
+    a byte-exact scatter, both written in C, with device memory and the stream from the harness hooks."""
+    import os
+    import subprocess
+    client = os.path.join(os.path.dirname(rt.IMPL_LIB_PATH), "diopi_c_client")
+    assert os.path.isfile(client), "the C host is built with the libraries"
+    res = subprocess.run([client], capture_output=True, text=True, timeout=120)
+    say(res.stdout)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "diopiRMSNorm fp32" in res.stdout and "bytes equal" in res.stdout and res.stdout.strip().endswith("c client ok")
+
+
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
