@@ -1148,6 +1148,100 @@ def test_decode_step_in_a_hip_graph_replays_like_eager():
         assert_close(got_out, ref, what=f"replay {replay}: decode output vs float64", **TOL[torch.float16])
 
 
+# ----------------------------------------------------------------------------- tensors past 2^31 elements
+def test_tensors_with_more_than_two_to_the_31_elements():
+    """64-bit addressing: every large tensor here holds 2^31 + 20480 elements (4 GiB of bf16).  Results are compared
+    with the oracle on the first, middle and last rows and a random sample, which is where a 32-bit offset would wrap.
+    Covers both normalisations, rotary, the cache scatter, the two decode operators and the prefill operator."""
+    dt = torch.bfloat16
+    rows, H, D = 2 ** 19 + 5, 32, 128
+    n2 = H * D
+    assert rows * n2 > 2 ** 31
+    g = gen(900)
+    x = torch.empty(rows, n2, dtype=dt, device=DEV).normal_()
+    res = torch.empty(rows, n2, dtype=dt, device=DEV).normal_()
+    out = torch.empty(rows, n2, dtype=dt, device=DEV)
+    wt = (torch.rand(n2, generator=g) + 0.5).to(dt).to(DEV)
+    pick = torch.cat((torch.tensor([0, 1, rows // 2, rows - 2, rows - 1]), torch.randint(0, rows, (27,), generator=g))).to(DEV)
+    xs, rs = x[pick].cpu(), res[pick].cpu()
+
+    say("past 2^31: rms_norm")
+    o = F.rms_norm(x, (n2,), wt, None, 1e-6)
+    want, want_inv = O.rms_norm(xs, (n2,), wt.cpu(), None, 1e-6)
+    assert_close(o[pick], want, what="rms_norm past 2^31", **TOL[dt])
+    assert_close(F.GLOBAL_STATE["rms_norm_inv_rms"][pick], want_inv, rtol=1e-5, atol=0, what="inv_rms past 2^31")
+    del o
+
+    say("past 2^31: rotary")
+    cos = torch.randn(rows, 1, D // 2, generator=g).to(dt).to(DEV)
+    sin = torch.randn(rows, 1, D // 2, generator=g).to(dt).to(DEV)
+    ro = F.rotary_emb(x.view(rows, H, D), cos, sin, False, False)
+    assert_close(ro[pick], O.rotary_emb(xs.view(-1, H, D), cos[pick].cpu(), sin[pick].cpu(), False), what="rotary past 2^31", **TOL[dt])
+    del ro
+
+    say("past 2^31: fused residual addition + normalisation, in place")
+    out.copy_(x)
+    F.fused_add_root_mean_square_norm_inp(out, res, None, wt, 1e-6)
+    w_out, w_res = O.fused_add_root_mean_square_norm_inp(xs, rs, None, wt.cpu(), 1e-6)
+    assert_bit_equal(res[pick], w_res, "fused norm past 2^31: residual")
+    assert_close(out[pick], w_out, what="fused norm past 2^31", **TOL[dt])
+
+    say("past 2^31: destindex_copy_kv")
+    cache = out.view(rows, H, D)
+    dest = torch.tensor([rows - 1, 0, rows - 3, rows // 2 + 1, 7, rows - 2], dtype=torch.int64, device=DEV)
+    newk = torch.randn(6, H, D, generator=g).to(dt).to(DEV)
+    others = pick[~torch.isin(pick, dest)]
+    untouched = cache[others].clone()
+    F.destindex_copy_kv(newk, dest, cache)
+    assert_bit_equal(cache[dest], newk, "destindex past 2^31: scattered rows")
+    assert_bit_equal(cache[others], untouched, "destindex past 2^31: other rows")
+
+    say("past 2^31: decode over slots at the top of the cache")
+    kc, vc = x.view(rows, H, D), res.view(rows, H, D)
+    lens = [300, 77]
+    maxlen = 320
+    b_loc = torch.zeros(2, maxlen, dtype=torch.int32)
+    top = torch.randperm(4096, generator=g)[: sum(lens)]
+    used = rows - 1 - top  # distinct slots among the last 4096 rows
+    b_loc[0, maxlen - lens[0]:] = used[: lens[0]].int()
+    b_loc[1, maxlen - lens[1]:] = used[lens[0]:].int()
+    b_seq = torch.tensor(lens, dtype=torch.int32)
+    b_start = torch.tensor([0, lens[0]], dtype=torch.int32)
+    q = torch.randn(2, H, D, generator=g).to(dt)
+    logits = torch.zeros(H, sum(lens), dtype=dt, device=DEV)
+    F.token_attention(q.to(DEV), kc, logits, b_loc.to(DEV), b_start.to(DEV), b_seq.to(DEV), maxlen)
+    o2 = torch.zeros(2, H, D, dtype=dt, device=DEV)
+    F.token_softmax_reducev(logits, vc, o2, b_loc.to(DEV), b_start.to(DEV), b_seq.to(DEV), maxlen, 0)
+    # the oracle sees a compact cache that holds only the used rows, through a row table renumbered to match
+    order = used.sort().values
+    small_k, small_v = kc[order.to(DEV)].cpu(), vc[order.to(DEV)].cpu()
+    remap = torch.zeros_like(b_loc)
+    live = torch.zeros_like(b_loc, dtype=torch.bool)
+    live[0, maxlen - lens[0]:] = True
+    live[1, maxlen - lens[1]:] = True
+    remap[live] = torch.searchsorted(order, b_loc[live].long()).int()
+    want_logits = O.token_attention(q, small_k, torch.zeros(H, sum(lens), dtype=dt), remap, b_start, b_seq, maxlen)
+    assert_close(logits, want_logits, what="token_attention past 2^31", **TOL[dt])
+    want_o = O.token_softmax_reducev(logits.cpu(), small_v, torch.zeros(2, H, D, dtype=dt), remap, b_start, b_seq, maxlen, 0)
+    assert_close(o2, want_o, what="token_softmax_reducev past 2^31", **TOL[dt])
+
+    say("past 2^31: prefill over sequences at both ends and in the middle of the token axis")
+    starts, plens = [0, rows // 2, rows - 300], [200, 257, 300]
+    qv, kv, vv = x.view(rows, H, D), res.view(rows, H, D), out.view(rows, H, D)
+    ctx_out = torch.full((rows, H, D), 7.0, dtype=dt, device=DEV)
+    F.context_attention(qv, kv, vv, ctx_out, torch.tensor(starts, dtype=torch.int32, device=DEV), torch.tensor(plens, dtype=torch.int32, device=DEV),
+                        max(plens))
+    for st, ln in zip(starts, plens):
+        sl = slice(st, st + ln)
+        # against the float64 evaluation: the kernel keeps its scores in fp32, and with unit-variance bf16 inputs the
+        # reference's rounding of the scores to bf16 alone moves single outputs by more than the bar
+        want_c = O.context_attention(qv[sl].cpu(), kv[sl].cpu(), vv[sl].cpu(), torch.zeros(ln, H, D, dtype=torch.float64), torch.tensor([0]),
+                                     torch.tensor([ln]), exact=True)
+        assert_close(ctx_out[sl], want_c, what=f"context_attention past 2^31, rows {st}..{st + ln}", **TOL[dt])
+    outside = torch.tensor([200, 201, rows // 2 - 1, rows // 2 + 257, rows - 301, 12345], device=DEV)
+    assert bool((ctx_out[outside] == 7.0).all()), "rows outside every sequence were written"
+
+
 # ----------------------------------------------------------------------------- the reference harness's device hooks
 def test_harness_hooks_drive_an_operator_without_torch_on_the_device():
     """The way diopi_test reaches the device (conform_test.h:28-43; litert.cpp:370-376): memory from device_malloc,
