@@ -1152,7 +1152,7 @@ def test_decode_step_in_a_hip_graph_replays_like_eager():
 def test_tensors_with_more_than_two_to_the_31_elements():
     """64-bit addressing: every large tensor here holds 2^31 + 20480 elements (4 GiB of bf16).  Results are compared
     with the oracle on the first, middle and last rows and a random sample, which is where a 32-bit offset would wrap.
-    Covers both normalisations, rotary, the cache scatter, the two decode operators and the prefill operator."""
+    Covers both normalisations and the backward pass, rotary, the cache scatter, the two decode operators and the prefill operator."""
     dt = torch.bfloat16
     rows, H, D = 2 ** 19 + 5, 32, 128
     n2 = H * D
@@ -1169,8 +1169,21 @@ def test_tensors_with_more_than_two_to_the_31_elements():
     o = F.rms_norm(x, (n2,), wt, None, 1e-6)
     want, want_inv = O.rms_norm(xs, (n2,), wt.cpu(), None, 1e-6)
     assert_close(o[pick], want, what="rms_norm past 2^31", **TOL[dt])
-    assert_close(F.GLOBAL_STATE["rms_norm_inv_rms"][pick], want_inv, rtol=1e-5, atol=0, what="inv_rms past 2^31")
+    inv_big = F.GLOBAL_STATE["rms_norm_inv_rms"]
+    assert_close(inv_big[pick], want_inv, rtol=1e-5, atol=0, what="inv_rms past 2^31")
     del o
+
+    say("past 2^31: rms_norm_backward")
+    grads = F.rms_norm_backward([res.view(rows, n2)], x, wt, None, (n2,), 1e-6, inv_rms=inv_big)
+    w_gi, _, _ = O.rms_norm_backward(rs, xs, wt.cpu(), inv_big[pick].cpu(), (n2,))
+    assert_close(grads["input"][pick], w_gi, what="grad_input past 2^31", **TOL[dt])
+    # grad_weight sums half a million rows: second opinion from float64 column sums formed on the device in slabs
+    col = torch.zeros(n2, dtype=torch.float64, device=DEV)
+    for lo in range(0, rows, 65536):
+        hi = min(rows, lo + 65536)
+        col += (res[lo:hi].double() * x[lo:hi].double() * inv_big[lo:hi].double()[:, None]).sum(0)
+    assert_close(grads["weight"], col.cpu(), rtol=1e-2, atol=1e-2 * math.sqrt(rows), what="grad_weight past 2^31")
+    del grads, col
 
     say("past 2^31: rotary")
     cos = torch.randn(rows, 1, D // 2, generator=g).to(dt).to(DEV)
