@@ -104,6 +104,29 @@ def test_destindex_copy_kv_edge_cases():
     assert_bit_equal(od, want, "empty scatter")
 
 
+def test_destindex_copy_kv_repeated_destinations():
+    """Several tokens sent to one row: the reference's non-accumulating index_put_ leaves the winner unspecified
+    (functions_lightllm.cpp:18-26).  Every element of such a row must come from one of the tokens sent there, rows that
+    receive one token get exactly that token, and all other rows stay as they were."""
+    g = gen(150)
+    for dt in (torch.float16, torch.float32):
+        k = torch.randn(64, 32, 128, generator=g).to(dt).to(DEV)
+        cache = torch.randn(40, 32, 128, generator=g).to(dt).to(DEV)
+        before = cache.clone()
+        dest = torch.tensor([3] * 20 + [7] * 30 + list(range(20, 33)) + [39], dtype=torch.int32, device=DEV)
+        F.destindex_copy_kv(k, dest, cache)
+        for row, senders in ((3, range(0, 20)), (7, range(20, 50))):
+            from_some_sender = torch.zeros(32, 128, dtype=torch.bool, device=DEV)
+            for t in senders:
+                from_some_sender |= cache[row].view(torch.int16 if dt == torch.float16 else torch.int32) == k[t].view(
+                    torch.int16 if dt == torch.float16 else torch.int32)
+            assert bool(from_some_sender.all()), f"row {row} holds bytes that none of its tokens carries"
+        assert_bit_equal(cache[20:33], k[50:63], "rows with a single token")
+        assert_bit_equal(cache[39], k[63], "last row")
+        rest = [r for r in range(40) if r not in (3, 7, 39) and not 20 <= r < 33]
+        assert_bit_equal(cache[rest], before[rest], "rows that no token was sent to")
+
+
 def test_destindex_copy_kv_large_round_trip():
     # encode -> scatter -> gather round trip over a full permutation of 65536 rows of 8 KiB
     T = 65536
