@@ -550,6 +550,27 @@ def test_decode_reference_fixture(golden, dtype):
     _decode_case(w, dt, f"decode fixture {dtype}")
 
 
+@pytest.mark.parametrize("dtype,Hq,Hkv", [("float16", 32, 32), ("bfloat16", 16, 2)])
+def test_decode_sequences_sharing_cache_rows(dtype, Hq, Hkv):
+    """Sequences with a common prefix point at the same cache rows (the row table is a table, not a partition): four
+    sequences share their first 600 rows and differ in their tails; one row table also names a row twice."""
+    dt = TORCH_DTYPES[dtype]
+    g = gen(560)
+    D, slots, maxlen = 128, 4096, 900
+    prefix = torch.randperm(slots, generator=g)[:600]
+    lens = [600, 731, 899, 655]
+    b_loc = torch.zeros(len(lens), maxlen, dtype=torch.int32)
+    for i, L in enumerate(lens):
+        tail = torch.randint(0, slots, (L - 600,), generator=g)
+        b_loc[i, maxlen - L:] = torch.cat((prefix, tail)).int()
+    b_loc[2, maxlen - 1] = b_loc[2, maxlen - 2]  # the same row twice in one sequence
+    starts = torch.tensor([0] + list(np.cumsum(lens)[:-1]), dtype=torch.int32)
+    w = dict(q=torch.randn(len(lens), Hq, D, generator=g).to(dt).to(DEV), k_cache=torch.randn(slots, Hkv, D, generator=g).to(dt).to(DEV),
+             v_cache=torch.randn(slots, Hkv, D, generator=g).to(dt).to(DEV), b_loc=b_loc.to(DEV), b_start_loc=starts.to(DEV),
+             b_seq_len=torch.tensor(lens, dtype=torch.int32, device=DEV), max_input_len=maxlen, total_len=sum(lens))
+    _decode_case(w, dt, f"decode with shared rows {dtype} {Hq}/{Hkv}")
+
+
 def test_decode_index_exactness_and_int64():
     # k[slot] = slot pattern: the logits are exact small integers times a constant, so any wrong slot shows up exactly
     D, H = 128, 32
