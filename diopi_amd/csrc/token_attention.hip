@@ -342,7 +342,9 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
     HS = envInt("DIOPI_ROCM_TOKATT_HS", HS);
     if (HS != 1 && HS != 2 && HS != 4) HS = 1;
-    int TT = envInt("DIOPI_ROCM_TOKATT_TT", 128);  // tokens per work-group
+    // tokens per work-group: with one query head per kv head, tiles of 64 tokens measured 1.7 % faster than 128 (64
+    // sequences of 512..2048 tokens, 32 heads); with 8 query heads per kv head 128 is 1.3 % faster than 64
+    int TT = envInt("DIOPI_ROCM_TOKATT_TT", a.G == 1 ? 64 : 128);
     TT = TT / 64 * 64;
     if (TT < 64) TT = 64;
     if (TT > 1024) TT = 1024;
