@@ -116,7 +116,8 @@ struct DeviceInfo {
 };
 const DeviceInfo& deviceInfo();
 
-// Integer knob from the environment (read once per name), for tuning experiments.
+// Integer knob from the environment, for tuning experiments: the variable is looked up once per name; when it is unset
+// every call gets its own fallback (fallbacks depend on the shapes of the call at hand).
 int envInt(const char* name, int fallback);
 
 inline int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

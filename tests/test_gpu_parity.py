@@ -571,6 +571,37 @@ def test_decode_sequences_sharing_cache_rows(dtype, Hq, Hkv):
     _decode_case(w, dt, f"decode with shared rows {dtype} {Hq}/{Hkv}")
 
 
+def test_decode_range_length_follows_each_call_not_the_first_one():
+    """The range length of the split decode kernel depends on the head grouping of the call at hand.  The scratch a call
+    asks for shows it: B * ceil(max_len / range) * H * (D + 2) * 4 bytes with range = max(256, 128 * G)."""
+    g = gen(570)
+    D, slots, maxlen, B = 128, 4096, 2048, 2
+
+    def scratch_of(Hq, Hkv):
+        ctx = rt.Context(own_stream=True)
+        q = torch.randn(B, Hq, D, generator=g).half().to(DEV)
+        v = torch.randn(slots, Hkv, D, generator=g).half().to(DEV)
+        b_loc = torch.stack([torch.randperm(slots, generator=g)[:maxlen] for _ in range(B)]).int().to(DEV)
+        lens = torch.tensor([maxlen, maxlen], dtype=torch.int32, device=DEV)
+        starts = torch.tensor([0, maxlen], dtype=torch.int32, device=DEV)
+        logits = torch.randn(Hq, B * maxlen, generator=g).half().to(DEV)
+        out = torch.zeros(B, Hq, D, dtype=torch.float16, device=DEV)
+        F.token_softmax_reducev(logits, v, out, b_loc, starts, lens, maxlen, 0, ctx=ctx)
+        ctx.synchronize()
+        peak = ctx.scratch_peak
+        ctx.close()
+        return peak
+
+    def expected(Hq, Hkv):
+        rng_len = max(256, 128 * (Hq // Hkv))
+        return B * math.ceil(maxlen / rng_len) * Hq * (D + 2) * 4
+
+    for Hq, Hkv in ((4, 4), (8, 1), (4, 4), (8, 2)):  # ungrouped first, then grouped, and back
+        peak = scratch_of(Hq, Hkv)
+        want = expected(Hq, Hkv)
+        assert want <= peak < want + 2048, f"{Hq}/{Hkv} heads: scratch {peak} bytes, expected {want} (+ rounding)"
+
+
 def test_decode_index_exactness_and_int64():
     # k[slot] = slot pattern: the logits are exact small integers times a constant, so any wrong slot shows up exactly
     D, H = 128, 32
