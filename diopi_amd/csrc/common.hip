@@ -265,6 +265,19 @@ const DeviceInfo& deviceInfo() {
     return info;
 }
 
+diopiError_t grantDynamicLds(const void* kernel, int bytes) {
+    static std::mutex mtx;
+    static std::map<std::pair<const void*, int>, int> granted;  // (kernel, device) -> bytes granted so far
+    int dev = 0;
+    ROCM_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mtx);
+    int& have = granted[std::make_pair(kernel, dev)];
+    if (have >= bytes) return diopiSuccess;
+    ROCM_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    have = bytes;
+    return diopiSuccess;
+}
+
 int envInt(const char* name, int fallback) {
     // what is remembered is the environment (set or not, and to what), never a caller's fallback: fallbacks depend
     // on the shapes of the call at hand

@@ -116,6 +116,10 @@ struct DeviceInfo {
 };
 const DeviceInfo& deviceInfo();
 
+// Lets `kernel` use `bytes` of dynamic LDS beyond the 64 KiB default, once per kernel and device (the attribute belongs
+// to the device the call runs on; a process may hold several).
+diopiError_t grantDynamicLds(const void* kernel, int bytes);
+
 // Integer knob from the environment, for tuning experiments: the variable is looked up once per name; when it is unset
 // every call gets its own fallback (fallbacks depend on the shapes of the call at hand).
 int envInt(const char* name, int fallback);

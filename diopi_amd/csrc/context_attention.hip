@@ -599,9 +599,7 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     const int grid = static_cast<int>(ceilDiv(total, kNumXcd)) * kNumXcd;
     constexpr int kStaging = 2 * 2 * kBN * kHD, kOutTile = BM * kLD;  // elements: two (K, V) buffers; the output tile that reuses them
     constexpr int ldsBytes = (kStaging > kOutTile ? kStaging : kOutTile) * static_cast<int>(sizeof(T));
-    static hipError_t granted =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV, GEN>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes);
-    ROCM_HIP(granted);
+    ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV, GEN>), ldsBytes));
     hipLaunchKernelGGL((ctxAttnMfma<T, NWV, GEN>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q),
                        static_cast<const T*>(k), static_cast<const T*>(v), a);
     ROCM_LAUNCH_CHECK();

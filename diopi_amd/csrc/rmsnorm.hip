@@ -662,16 +662,14 @@ diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const Tenso
 }
 
 // Launches one instantiation of the fused backward kernel; the LDS column-sum arrays are dynamic shared memory
-// beyond the 64 KiB static limit, which has to be granted per kernel once.
+// beyond the 64 KiB static limit, which has to be granted per kernel and device.
 template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS>
 diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, ColAcc* partW, ColAcc* partB, const T* dout, const T* in, const T* w,
                                const float* invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
     constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * kBwdTeam * EPV * sizeof(ColAcc);
     auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS>;
-    static hipError_t granted = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                    static_cast<int>(ldsBytes));
-    ROCM_HIP(granted);
+    ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(kernel), static_cast<int>(ldsBytes)));
     hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
