@@ -571,7 +571,7 @@ diopiError_t launchFwdFast(hipStream_t stream, const TensorView& out, const Tens
     if (d.n2 % EPV != 0 || d.n2 > INT32_MAX) return diopiSuccess;
     const int64_t nvec = d.n2 / EPV;
     if (nvec > 16 * kWave) return diopiSuccess;
-    if (!aligned16(in.data) || !aligned16(out.data) || !aligned16(w.data)) return diopiSuccess;
+    if (!aligned16(in.data) || !aligned16(out.data) || !aligned16(w.data) || !aligned16(bias)) return diopiSuccess;
     if (sizeof(TOut) != sizeof(TIn) && (reinterpret_cast<uintptr_t>(out.data) & 7) != 0) return diopiSuccess;
     const float feps = static_cast<float>(eps);
     const int n2 = static_cast<int>(d.n2);

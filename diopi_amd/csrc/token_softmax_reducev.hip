@@ -113,7 +113,19 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
     const int64_t t0 = static_cast<int64_t>(blockIdx.z) * sp.TT;
-    if (t0 >= L) return;
+    if (t0 >= L) {
+        // a sequence without tokens: the reference's product over an empty inner dimension gives zeros
+        // (functions_lightllm.cpp:98-104); the work-groups of range 0 write them
+        if (L <= 0 && blockIdx.z == 0) {
+            const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
+            const int hk0 = (blockIdx.x * kRvWaves + w) * HPW;
+            const int rows = (hk0 < a.Hkv) ? ((a.Hkv - hk0 < HPW ? a.Hkv - hk0 : HPW) * a.G) : 0;
+            Pack16<T> z;
+            z.raw = u32x4{0u, 0u, 0u, 0u};
+            for (int g = l / 16; g < rows; g += 4) storePack(out + (static_cast<int64_t>(i) * a.H + hk0 * a.G + g) * kD + (l % 16) * 8, z);
+        }
+        return;
+    }
     const int64_t tEnd = (t0 + sp.TT < L) ? t0 + sp.TT : L;
     const int nTokR = static_cast<int>(tEnd - t0);
     const int nSub = (nTokR + kSub - 1) / kSub;
@@ -382,11 +394,15 @@ __global__ __launch_bounds__(kRvThreads) void softmaxReduceVGeneric(T* __restric
     const int qh = blockIdx.x;
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    if (L <= 0) return;
+    const int tid = threadIdx.x;
+    if (L <= 0) {
+        // no tokens: zeros, as the reference's product over an empty inner dimension (functions_lightllm.cpp:98-104)
+        for (int d = tid; d < a.D; d += kRvThreads) out[(static_cast<int64_t>(i) * a.H + qh) * a.D + d] = static_cast<T>(0);
+        return;
+    }
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L);
     const T* row = logits + static_cast<int64_t>(qh) * a.logitCols;
-    const int tid = threadIdx.x;
     auto logitAt = [&](int64_t t) -> AccT {
         const int64_t col = start + t;
         return (col >= 0 && col < a.logitCols) ? static_cast<AccT>(row[col]) : static_cast<AccT>(-INFINITY);

@@ -48,6 +48,10 @@ class _on_stream:
     def __exit__(self, *exc):
         if self.cuda:
             torch.cuda.current_stream().wait_stream(self.ctx.torch_stream)
+        # scratch an operator took from the context (partial sums, tile plans, score buffers) belongs to that call:
+        # hand it back to the context's pool, as the reference harness does after every case (litert.hpp:268-276);
+        # the pool is reused in stream order, so a later call on this context may overwrite it safely
+        self.ctx.clear_tensors()
         return False
 
 
@@ -130,7 +134,6 @@ def rms_norm_backward(grad_outputs: Sequence[torch.Tensor], input: torch.Tensor,
     with _on_stream(ctx, input):
         keep, h = _handles(grad_input, grad_weight, grad_bias, grad_outputs[0], input, weight, bias, inv_rms)
         ret = rt.libs().impl.diopiRMSNormBackward(ctx.handle, *h, sizes.c, float(eps))
-    ctx.clear_tensors()
     check_returncode(ret, "diopiRMSNormBackward")
     out = {"input": grad_input, "weight": grad_weight}
     if bias is not None:
@@ -184,7 +187,6 @@ def token_softmax_reducev(logics: torch.Tensor, v: torch.Tensor, out: torch.Tens
     with _on_stream(ctx, out):
         keep, h = _handles(out, logics, v, b_loc, b_start_loc, b_seq_len)
         ret = rt.libs().impl.diopiTokenSoftmaxReduceVInference(ctx.handle, *h, int(max_input_len), int(other_kv_index))
-    ctx.clear_tensors()
     check_returncode(ret, "diopiTokenSoftmaxReduceVInference")
     return out
 
@@ -296,6 +298,5 @@ def paged_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
         keep, h = _handles(out, query, key, value, attenMask, blockTable)
         ret = rt.libs().impl.diopiPagedAttention(ctx.handle, h[0], h[1], h[2], h[3], h[4], sizes.c, int(numHeads), int(numKeyValueHeads), int(dim), h[5],
                                                  int(blockSize))
-    ctx.clear_tensors()
     check_returncode(ret, "diopiPagedAttention")
     return out

@@ -302,8 +302,8 @@ def token_softmax_reducev(logics: torch.Tensor, v: torch.Tensor, out: torch.Tens
     for i in range(batch):
         L = int(b_seq_len[i])
         s = int(b_start_loc[i])
-        if L == 0:
-            continue
+        # L == 0 is not skipped: the reference assigns the product over an empty inner dimension, i.e. zeros
+        # (functions_lightllm.cpp:98-104)
         v_loc = _window(b_loc, i, L, max_input_len)
         P = logics[:, s:s + L].to(cdt).softmax(-1).reshape(head, 1, 1, L).transpose(0, 1)  # [1, H, 1, L]
         V = v[v_loc].to(cdt)

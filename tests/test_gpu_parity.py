@@ -505,7 +505,7 @@ def _decode_case(w, dtype, what, seq_subset=None):
     logits = torch.full((H, total), -12288.0, dtype=dtype, device=DEV)
     before = snapshot(q, w["b_loc"], w["b_start_loc"], w["b_seq_len"])
     F.token_attention(q, kc, logits, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
-    out = torch.zeros_like(q)
+    out = torch.full_like(q, 7.0)  # every row must be written, also the zeros of a sequence without tokens
     F.token_softmax_reducev(logits, vc, out, w["b_loc"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], 0)
     assert_unmodified(before, q, w["b_loc"], w["b_start_loc"], w["b_seq_len"])
     idx = list(range(q.shape[0])) if seq_subset is None else seq_subset
@@ -528,9 +528,9 @@ def _decode_case(w, dtype, what, seq_subset=None):
     if seq_subset is None:
         assert_bit_equal(dev_logits, torch.where(ref_logits == -12288.0, ref_logits, dev_logits), what + ": columns outside every sequence were written")
     # second operator: feed the oracle the device's logits so that the two checks are independent
-    ref_out = torch.zeros(len(idx), H, q.shape[2], dtype=dtype)
+    ref_out = torch.full((len(idx), H, q.shape[2]), -3.0, dtype=dtype)
     O.token_softmax_reducev(dev_logits, v_small, ref_out, loc_small, b_start_c, b_len_c, w["max_input_len"], 0)
-    ex_out = torch.zeros(len(idx), H, q.shape[2], dtype=torch.float64)
+    ex_out = torch.full((len(idx), H, q.shape[2]), -3.0, dtype=torch.float64)
     O.token_softmax_reducev(dev_logits, v_small, ex_out, loc_small, b_start_c, b_len_c, w["max_input_len"], 0, exact=True)
     assert_close(out.cpu()[sel], ref_out, what=what + " out vs reference composition", **tol)
     assert_close(out.cpu()[sel], ex_out, what=what + " out vs float64", **tol)
@@ -644,6 +644,45 @@ def test_decode_gqa_config5_scaled():
     for G, Hkv in ((2, 4), (4, 2), (16, 1), (3, 2)):
         w3 = W._decode(DEV, 55 + G, torch.float16, 3, G * Hkv, Hkv, 128, 2048, 5, 600, 3)
         _decode_case(w3, torch.float16, f"GQA G={G} Hkv={Hkv}")
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_decode_head_size_64(dtype):
+    """Head size 64 takes the matrix-core kernel that reads its operands straight from the cache rows (score operator)
+    and the shape-agnostic reduce kernel: one query head per cache head and grouped heads, ragged lengths that are no
+    multiple of 16 or 128 (and an empty sequence), 32- and 64-bit index tensors."""
+    dt = TORCH_DTYPES[dtype]
+    for (H, Hkv, idt) in ((8, 8, torch.int32), (12, 3, torch.int64), (16, 1, torch.int32)):
+        lens = np.array([1, 15, 16, 17, 0, 127, 128, 129, 300, 77], dtype=np.int64)
+        B = len(lens)
+        w = W._decode(DEV, 640 + H, dt, B, H, Hkv, 64, 4096, 1, 320, B)
+        w["b_seq_len"] = torch.from_numpy(lens).to(idt).to(DEV)
+        w["b_start_loc"] = torch.from_numpy(np.concatenate(([0], np.cumsum(lens)[:-1]))).to(idt).to(DEV)
+        w["b_loc"] = w["b_loc"].to(idt)
+        w["total_len"] = int(lens.sum())
+        w["max_input_len"] = 310
+        _decode_case(w, dt, f"decode D=64 {dtype} H={H} Hkv={Hkv} {idt}")
+
+
+def test_context_attention_scratch_returns_to_the_pool():
+    """The tile plan of a prefill call is context scratch: repeated calls through the Python wrappers must reuse one
+    block of the context's pool instead of growing it."""
+    g = gen(641)
+    T = 700
+    q, k, v = ((torch.randn(T, 2, 128, generator=g) * 0.5).half().to(DEV) for _ in range(3))
+    bs, bl = torch.tensor([0, 300], dtype=torch.int32, device=DEV), torch.tensor([300, 400], dtype=torch.int32, device=DEV)
+    ctx = rt.Context(own_stream=True)
+    out = torch.zeros_like(q)
+    F.context_attention(q, k, v, out, bs, bl, 400, ctx=ctx)
+    first = ctx.malloc_count
+    assert first == 1
+    for _ in range(20):
+        F.context_attention(q, k, v, out, bs, bl, 400, ctx=ctx)
+        F.flash_attention_varlen(q, k, v, torch.tensor([0, 300, 700], dtype=torch.int32, device=DEV), torch.tensor([0, 300, 700], dtype=torch.int32, device=DEV),
+                                 None, 400, 400, 0.0, None, True, ctx=ctx)
+    ctx.synchronize()
+    assert ctx.malloc_count == first, f"the pool grew: {ctx.malloc_count} allocations"
+    ctx.close()
 
 
 def test_decode_config3_full_size_sampled():

@@ -442,6 +442,20 @@ def test_softmax_reducev_brute_force(G):
             assert np.allclose(out[i, h].numpy(), acc, rtol=1e-13, atol=1e-14)
 
 
+def test_softmax_reducev_sequence_without_tokens_gives_zeros():
+    """functions_lightllm.cpp:98-104 assigns out[i] for every i: with L = 0 the product has an empty inner dimension,
+    whose value is zero whatever the row held before; the neighbours are unaffected."""
+    g = rng(12)
+    v = torch.randn(20, 2, 8, generator=g).half()
+    b_loc = torch.stack([torch.randperm(20, generator=g)[:6] for _ in range(3)]).int()
+    logits = torch.randn(2, 7, generator=g).half()
+    for exact in (False, True):
+        out = torch.full((3, 2, 8), 9.0, dtype=torch.float64 if exact else torch.float16)
+        O.token_softmax_reducev(logits, v, out, b_loc, torch.tensor([0, 4, 4]), torch.tensor([4, 0, 3]), 5, 0, exact=exact)
+        assert bool((out[1] == 0).all()), "an empty sequence must produce zeros"
+        assert bool((out[0] != 9.0).all()) and bool((out[2] != 9.0).all())
+
+
 # ----------------------------------------------------------------------------- context_attention
 def _brute_context(q, k, v, start, L):
     H, D = q.shape[1], q.shape[2]
