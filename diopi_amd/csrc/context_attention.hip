@@ -33,6 +33,7 @@
 // second output.  That form is a template flag (GEN): the lightllm operator keeps its literal scale and its
 // compile-time causal structure.
 #include <cmath>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -68,6 +69,18 @@ struct CtxArgs {
     float* lse;        // [batch, H, lseStride] log-sum-exp of the scaled scores of every query row, or null
     int lseStride;     // max_seqlen_q
 };
+
+// Where a call keeps its tile plan: in scratch of the caller's context (the default), or in the library's own static
+// device array (the allocation-free entry point).
+struct PlanStore {
+    int4* fixed = nullptr;  // device address of the static array on the current device, or null: ask the context
+    int capacity = 0;       // entries of the static array
+};
+
+// Tile plans of the allocation-free entry point.  One array per device the library runs on, held until the process
+// ends; every call on a device shares it, so such calls must not overlap on one device.
+constexpr int kStaticPlanEntries = 8192;  // 128 KiB: query tiles + sequences of one call
+static __device__ __align__(256) int4 scratch[kStaticPlanEntries];
 
 template <typename T>
 struct Mfma32;
@@ -582,15 +595,23 @@ __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, con
 }
 
 template <typename T, int NWV, bool GEN = false>
-diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a) {
+diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* q, const void* k, const void* v, CtxArgs a,
+                        const PlanStore& store) {
     constexpr int BM = NWV * 32;
     a.tilesBound = static_cast<int>(ceilDiv(a.rows, BM)) + a.batch;
     const int64_t total = static_cast<int64_t>(a.tilesBound) * a.H;
     ROCM_CHECK(total < INT32_MAX / 2, "context attention: too many tiles for one launch");
     a.totalItems = static_cast<int>(total);
-    // visiting order of the query tiles (context-owned scratch, rebuilt by every call on the device)
-    void* planMem = nullptr;
-    ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int4), &planMem));
+    // visiting order of the query tiles, rebuilt by every call on the device: context-owned scratch, or the library's
+    // static array when the caller must not allocate
+    void* planMem = store.fixed;
+    if (store.fixed != nullptr) {
+        ROCM_CHECK(a.tilesBound <= store.capacity,
+                   "the allocation-free entry point holds a plan of at most %d query tiles of %d rows (+ one per sequence); this call needs %d",
+                   store.capacity, BM, a.tilesBound);
+    } else {
+        ROCM_CALL(requireScratch(ctx, static_cast<int64_t>(a.tilesBound) * sizeof(int4), &planMem));
+    }
     a.plan = static_cast<const int4*>(planMem);
     const int maxTiles = static_cast<int>(ceilDiv(a.rows, BM));
     const size_t planLds = (4 * static_cast<size_t>(a.batch) + maxTiles) * sizeof(int);
@@ -623,7 +644,7 @@ diopiError_t launchGeneric(hipStream_t stream, void* out, const void* q, const v
 // for everything else.  Returns diopiDtypeNotSupported (without a message) for a dtype no kernel takes.
 template <bool GEN>
 diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, const TensorView& vOut, const TensorView& vQ, const TensorView& vK,
-                               const TensorView& vV, const CtxArgs& a, int D, double softmaxScale) {
+                               const TensorView& vV, const CtxArgs& a, int D, double softmaxScale, const PlanStore& store = PlanStore()) {
     const bool aligned =
         ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data) | reinterpret_cast<uintptr_t>(vV.data) | reinterpret_cast<uintptr_t>(vOut.data)) & 15) == 0;
     // the planning kernel keeps two ints per sequence and one per query tile in LDS
@@ -635,12 +656,12 @@ diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, con
     const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
     switch (vQ.dtype) {
         case diopi_dtype_float16:
-            return fast ? (wide ? launchMfma<half_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
-                                : launchMfma<half_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
+            return fast ? (wide ? launchMfma<half_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a, store)
+                                : launchMfma<half_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a, store))
                         : launchGeneric<half_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
         case diopi_dtype_bfloat16:
-            return fast ? (wide ? launchMfma<bf16_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a)
-                                : launchMfma<bf16_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a))
+            return fast ? (wide ? launchMfma<bf16_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a, store)
+                                : launchMfma<bf16_t, 4, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a, store))
                         : launchGeneric<bf16_t, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
         case diopi_dtype_float32: return launchGeneric<float, float>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
         case diopi_dtype_float64: return launchGeneric<double, double>(stream, vOut.data, vQ.data, vK.data, vV.data, a, D, softmaxScale);
@@ -652,12 +673,35 @@ diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, con
 }  // namespace
 }  // namespace rocm
 
-extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
-                                                       diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
-                                                       diopiConstTensorHandle_t b_seq_len, int max_input_len) {
-    ROCM_ENTRY_BEGIN
-    using namespace rocm;
-    (void)max_input_len;  // never read by the reference (functions_lightllm.cpp:127-147); lengths come from b_seq_len
+namespace rocm {
+namespace {
+
+// Device address of the static plan array on the current device.  In host code the array's name is only a stand-in
+// for the symbol; the address a kernel may use comes from hipGetSymbolAddress, once per device (each device holds its
+// own copy at its own address).
+diopiError_t staticPlanStore(PlanStore* store) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mtx;
+    static int4* address[kMaxDevices] = {nullptr};
+    int dev = 0;
+    ROCM_HIP(hipGetDevice(&dev));
+    ROCM_CHECK(dev >= 0 && dev < kMaxDevices, "device index %d is beyond the %d devices the allocation-free entry point keeps a plan for", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(mtx);
+    if (address[dev] == nullptr) {
+        void* ptr = nullptr;
+        ROCM_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        ROCM_CHECK(ptr != nullptr, "hipGetSymbolAddress returned no address for the static plan array");
+        address[dev] = static_cast<int4*>(ptr);
+    }
+    store->fixed = address[dev];
+    store->capacity = kStaticPlanEntries;
+    return diopiSuccess;
+}
+
+// diopiContextAttentionInference and its allocation-free variant: the same checks and kernels, the tile plan in the
+// context's scratch (`staticPlan` false) or in the library's static array.
+diopiError_t contextAttention(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q, diopiConstTensorHandle_t k,
+                              diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc, diopiConstTensorHandle_t b_seq_len, bool staticPlan) {
     TensorView vOut, vQ, vK, vV, vStart, vLen;
     ROCM_CALL(unwrap(context_attention_out, "context_attention_out", &vOut));
     ROCM_CALL(unwrap(q, "q", &vQ));
@@ -700,10 +744,37 @@ extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx,
     const int D = static_cast<int>(vQ.shape[2]);
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    const diopiError_t err = dispatchAttention<false>(ctx, stream, vOut, vQ, vK, vV, a, D, 1.0 / std::sqrt(static_cast<double>(D)));
+    PlanStore store;
+    if (staticPlan) ROCM_CALL(staticPlanStore(&store));
+    const diopiError_t err = dispatchAttention<false>(ctx, stream, vOut, vQ, vK, vV, a, D, 1.0 / std::sqrt(static_cast<double>(D)), store);
     if (err != diopiDtypeNotSupported) return err;
     setLastError("diopiContextAttentionInference: dtype %s is not supported", dtypeName(vQ.dtype));
     return diopiDtypeNotSupported;
+}
+
+}  // namespace
+}  // namespace rocm
+
+extern "C" diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
+                                                       diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
+                                                       diopiConstTensorHandle_t b_seq_len, int max_input_len) {
+    ROCM_ENTRY_BEGIN
+    (void)max_input_len;  // never read by the reference (functions_lightllm.cpp:127-147); lengths come from b_seq_len
+    return rocm::contextAttention(ctx, context_attention_out, q, k, v, b_start_loc, b_seq_len, false);
+    ROCM_ENTRY_END
+}
+
+// The same operator for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+// forbid hipMalloc): it calls neither diopiRequireBuffer / diopiRequireTensor nor any allocating routine.  The tile
+// plan lives in a static device array of kStaticPlanEntries entries that all such calls on one device share: calls
+// that overlap on one device (two streams) race on it.  Nothing in it has to start at zero: the planning kernel
+// rewrites every entry a call reads.  Inputs beyond the array's capacity are rejected with an error.
+extern "C" diopiError_t diopiContextAttentionInferenceNoAlloc(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out,
+                                                              diopiConstTensorHandle_t q, diopiConstTensorHandle_t k, diopiConstTensorHandle_t v,
+                                                              diopiConstTensorHandle_t b_start_loc, diopiConstTensorHandle_t b_seq_len, int max_input_len) {
+    ROCM_ENTRY_BEGIN
+    (void)max_input_len;
+    return rocm::contextAttention(ctx, context_attention_out, q, k, v, b_start_loc, b_seq_len, true);
     ROCM_ENTRY_END
 }
 

@@ -201,6 +201,18 @@ def context_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: to
     return out
 
 
+def context_attention_no_alloc(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor,
+                               max_input_len: int, ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """context_attention through the entry point that allocates nothing (no counterpart in the reference): the tile plan
+    lives in a static device array of the library, so calls on one device must not overlap."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, out):
+        keep, h = _handles(out, q, k, v, b_start_loc, b_seq_len)
+        ret = rt.libs().impl.diopiContextAttentionInferenceNoAlloc(ctx.handle, *h, int(max_input_len))
+    check_returncode(ret, "diopiContextAttentionInferenceNoAlloc")
+    return out
+
+
 def flash_attention_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_kv: torch.Tensor, alibi_slopes,
                            max_seqlen_q: int, max_seqlen_kv: int, p_dropout: float, softmax_scale, is_causal: bool, window_size_left: int = -1,
                            window_size_right: int = -1, ctx: Optional[rt.Context] = None) -> torch.Tensor:

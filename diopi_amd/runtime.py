@@ -161,6 +161,7 @@ class _Libs:
         impl.diopiTokenAttentionInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
         impl.diopiTokenSoftmaxReduceVInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32, i32]
         impl.diopiContextAttentionInference.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
+        impl.diopiContextAttentionInferenceNoAlloc.argtypes = [vp, vp, vp, vp, vp, vp, vp, i32]
         impl.diopiFlashAttentionVarLen.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, ctypes.c_float, ctypes.c_float, ctypes.c_bool,
                                                    i32, i32]
         impl.diopiFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_float, ctypes.c_float, ctypes.c_bool, i32, i32]
@@ -187,6 +188,7 @@ OPERATOR_SYMBOLS = (
     "diopiTokenAttentionInference",
     "diopiTokenSoftmaxReduceVInference",
     "diopiContextAttentionInference",
+    "diopiContextAttentionInferenceNoAlloc",
     "diopiFlashAttentionVarLen",
     "diopiFlashAttention",
     "diopiMultiHeadAttention",

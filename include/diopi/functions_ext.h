@@ -141,6 +141,20 @@ DIOPI_API diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, 
                                                       diopiConstTensorHandle_t b_seq_len, int max_input_len);
 
 /*
+ * diopiContextAttentionInference for callers that cannot allocate.
+ * No counterpart in the reference: this entry point exists for code that runs under HIP graph capture, tight serving
+ * loops and harnesses that forbid hipMalloc.  Same arguments, checks and results as diopiContextAttentionInference,
+ * but it never calls diopiRequireBuffer / diopiRequireTensor or any other allocating routine: the visiting order of
+ * the query tiles is kept in a static device array of the library (128 KiB per device, held until the process ends).
+ * Limit: ceil(rows / BM) + batch <= 8192 (BM = 256 query rows once the sequences average 1024 rows or more, else
+ * 128); a larger call returns diopiErrorOccurred with a message.  All calls on one device share the array: calls that
+ * overlap on one device (different streams or threads) race on it and must be serialised by the caller.
+ */
+DIOPI_API diopiError_t diopiContextAttentionInferenceNoAlloc(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
+                                                             diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,
+                                                             diopiConstTensorHandle_t b_seq_len, int max_input_len);
+
+/*
  * Variable-length flash attention, forward.
  * reference: functions_ext.h:355-359 (Python statement customized_test.py:525-588, 36-57).
  * q [total, Hq, D]; k, v [total, Hkv, D] with Hq a multiple of Hkv (query head h reads key/value head h / (Hq/Hkv));
