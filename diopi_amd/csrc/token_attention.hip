@@ -169,8 +169,15 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttMfma(T* __restrict__ out,
 //     first use; each [16 tokens x 128 dims] block then goes through a wave-private LDS tile
 //     (row pitch 272 bytes: conflict-free for both the 16-byte row writes and the 16-byte
 //     column-block reads) and comes back in the MFMA B-operand layout;
-//   * LDS operations of one wave execute in order, so the private tile needs no barrier.
+//   * LDS operations of one wave execute in order, so the private tile needs no barrier;
+//   * the scores of the whole tile wait in LDS, one line per query head, and the work-group writes them out at the end
+//     in 16-byte packets along the token axis (the MFMA result layout would send every wave store to two or four
+//     far-apart 32-byte pieces of the logits).
 // Waves are mapped to (head slot, token phase): with few kv heads the spare waves take other units.
+// What bounds this kernel when several query heads share a kv head is the logits themselves: on 128 sequences of
+// 1024..8192 tokens, 8 kv heads and 8 query heads each, the rows alone stream in 176 us, and the 6 % of the bytes
+// that are logits add 60..75 us whatever their layout, cache policy or place in the instruction stream (a copy of this
+// kernel's access pattern without arithmetic shows the same).
 constexpr int kStagePitch = 136;  // elements per staged row: 128 + 8
 
 template <typename T, int HW>
@@ -185,6 +192,7 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     constexpr int NG = TU / 16;   // MFMA column groups per unit
     __shared__ __attribute__((aligned(16))) T stage[kAttWaves][16 * kStagePitch];
     __shared__ int sSlot[1024];   // slot index of every token of the tile (TT <= 1024)
+    extern __shared__ __attribute__((aligned(16))) unsigned char dynLds[];  // scores of the tile: HS*HW*G rows of TT + 8
 
     // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
     // time), y over sequences, z over token tiles, with the sequence rotated by the tile index so that consecutive
@@ -213,64 +221,111 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     const int TPH = kAttWaves / HS;
     const int hs = wave % HS;
     const int tph = wave / HS;
-    const int hk0 = (blockIdx.x * HS + hs) * HW;
-    if (hk0 >= a.Hkv) return;
+    const int hkGroup = blockIdx.x * HS * HW;  // first kv head of the work-group
+    const int hk0 = hkGroup + hs * HW;
     const int64_t rowStride = static_cast<int64_t>(a.Hkv) * D;
     T* myStage = stage[wave];
 
-    // A fragments of this wave's heads: row c is query head (hk0+u)*G + c, k slot (r, e) <-> dim 32*s + 8*r + e
-    Frag qa[HW][KSTEPS];
-#pragma unroll
-    for (int u = 0; u < HW; ++u) {
-#pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) {
-            const bool valid = c < a.G && hk0 + u < a.Hkv;
-            qa[u][s] = valid ? loadFrag<Frag>(q + (static_cast<int64_t>(i) * a.H + (hk0 + u) * a.G + c) * D + s * 32 + r * 8) : zeroFrag<Frag>();
-        }
-    }
+    // The scores of the tile are collected in LDS, one row per query head, and written out afterwards in 16-byte
+    // packets along the token axis: the MFMA result layout would send every wave store to two or four far-apart
+    // 32-byte pieces.  Element t of local row j sits at sOut[j * outPitch + mis(j) + t], where mis(j) is the offset
+    // of the row's first logits element inside its 16-byte packet in global memory, so that packets of the LDS row
+    // and packets of the logits row coincide.
+    T* sOut = reinterpret_cast<T*>(dynLds);
+    const int outPitch = TT + 8;  // (TT + 8) / 2 banks: 4 rows apart is 16 banks apart for TT a multiple of 64
+    const int64_t col0 = start + t0;
+    const int64_t elem0 = static_cast<int64_t>(reinterpret_cast<uintptr_t>(out) / sizeof(T)) + col0;
 
-    const int numUnits = (nTok + TU - 1) / TU;
-    for (int unit = tph; unit < numUnits; unit += TPH) {
-        const int tu0 = unit * TU;
-        // every load of the unit is issued before the first use
-        u32x4 kv[NJ][HW];
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const int64_t rowOff = static_cast<int64_t>(sSlot[tu0 + 4 * j + r]) * rowStride;
-#pragma unroll
-            for (int u = 0; u < HW; ++u) {
-                const int hk = (hk0 + u < a.Hkv) ? hk0 + u : a.Hkv - 1;
-                kv[j][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k + rowOff + hk * D + c * 8));
-            }
-        }
+    if (hk0 < a.Hkv) {
+        // A fragments of this wave's heads: row c is query head (hk0+u)*G + c, k slot (r, e) <-> dim 32*s + 8*r + e
+        Frag qa[HW][KSTEPS];
 #pragma unroll
         for (int u = 0; u < HW; ++u) {
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                // 16 tokens x 128 dims of head u: rows 4*jj + r of the private tile
+            for (int s = 0; s < KSTEPS; ++s) {
+                const bool valid = c < a.G && hk0 + u < a.Hkv;
+                qa[u][s] = valid ? loadFrag<Frag>(q + (static_cast<int64_t>(i) * a.H + (hk0 + u) * a.G + c) * D + s * 32 + r * 8) : zeroFrag<Frag>();
+            }
+        }
+        // where this lane's four result rows (query heads 4*r + rr of head u) start in sOut
+        int outBase[HW][4];
 #pragma unroll
-                for (int jj = 0; jj < 4; ++jj) *reinterpret_cast<u32x4*>(myStage + (4 * jj + r) * kStagePitch + c * 8) = kv[4 * g + jj][u];
-                __builtin_amdgcn_wave_barrier();  // keep the tile writes ahead of the reads in program order
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < HW; ++u) {
 #pragma unroll
-                for (int s = 0; s < KSTEPS; ++s) {
-                    const Frag kb = loadFrag<Frag>(myStage + c * kStagePitch + s * 32 + r * 8);
-                    acc = Ops::mma(qa[u][s], kb, acc);
+            for (int rr = 0; rr < 4; ++rr) {
+                const int j = (hs * HW + u) * a.G + 4 * r + rr;
+                const int64_t hq = static_cast<int64_t>(hk0 + u) * a.G + 4 * r + rr;
+                outBase[u][rr] = j * outPitch + static_cast<int>((elem0 + hq * a.logitCols) & 7);
+            }
+        }
+
+        const int numUnits = (nTok + TU - 1) / TU;
+        for (int unit = tph; unit < numUnits; unit += TPH) {
+            const int tu0 = unit * TU;
+            // every load of the unit is issued before the first use
+            u32x4 kv[NJ][HW];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int64_t rowOff = static_cast<int64_t>(sSlot[tu0 + 4 * j + r]) * rowStride;
+#pragma unroll
+                for (int u = 0; u < HW; ++u) {
+                    const int hk = (hk0 + u < a.Hkv) ? hk0 + u : a.Hkv - 1;
+                    kv[j][u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k + rowOff + hk * D + c * 8));
                 }
-                __builtin_amdgcn_wave_barrier();  // ... and the reads ahead of the next tile's writes
-                // C: this lane holds query heads 4*r + rr of token column c
-                const int t = tu0 + g * 16 + c;
-                const int64_t col = start + t0 + t;
-                if (t < nTok && hk0 + u < a.Hkv && col >= 0 && col < a.logitCols) {
+            }
 #pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) {
-                        const int gh = 4 * r + rr;
-                        if (gh < a.G) {
-                            const T dot = static_cast<T>(acc[rr]);
-                            out[static_cast<int64_t>((hk0 + u) * a.G + gh) * a.logitCols + col] = static_cast<T>(static_cast<float>(dot) * scale);
+            for (int u = 0; u < HW; ++u) {
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    // 16 tokens x 128 dims of head u: rows 4*jj + r of the private tile
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) *reinterpret_cast<u32x4*>(myStage + (4 * jj + r) * kStagePitch + c * 8) = kv[4 * g + jj][u];
+                    __builtin_amdgcn_wave_barrier();  // keep the tile writes ahead of the reads in program order
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < KSTEPS; ++s) {
+                        const Frag kb = loadFrag<Frag>(myStage + c * kStagePitch + s * 32 + r * 8);
+                        acc = Ops::mma(qa[u][s], kb, acc);
+                    }
+                    __builtin_amdgcn_wave_barrier();  // ... and the reads ahead of the next tile's writes
+                    // C: this lane holds query heads 4*r + rr of token column c
+                    const int t = tu0 + g * 16 + c;
+                    if (hk0 + u < a.Hkv) {
+#pragma unroll
+                        for (int rr = 0; rr < 4; ++rr) {
+                            if (4 * r + rr < a.G) {
+                                const T dot = static_cast<T>(acc[rr]);
+                                sOut[outBase[u][rr] + t] = static_cast<T>(static_cast<float>(dot) * scale);
+                            }
                         }
                     }
                 }
+            }
+        }
+    }
+    __syncthreads();
+
+    // write-out: local row j is query head hkGroup*G + j; columns outside the logits tensor are dropped
+    const int rowsHere = ((hkGroup + HS * HW < a.Hkv) ? HS * HW : a.Hkv - hkGroup) * a.G;
+    int tLo = 0, tHi = nTok;
+    if (col0 < 0) tLo = static_cast<int>(-col0 < nTok ? -col0 : nTok);
+    if (col0 + nTok > a.logitCols) tHi = static_cast<int>(a.logitCols - col0 > 0 ? a.logitCols - col0 : 0);
+    const int packets = (TT + 8) / 8;
+    for (int item = threadIdx.x; item < rowsHere * packets; item += kAttThreads) {
+        const int j = item / packets;
+        const int p = item - j * packets;
+        const int64_t rowElem = (static_cast<int64_t>(hkGroup) * a.G + j) * a.logitCols + col0;  // of token 0 of the tile
+        const int mis = static_cast<int>((elem0 + (static_cast<int64_t>(hkGroup) * a.G + j) * a.logitCols) & 7);
+        const int tFirst = 8 * p - mis;  // token of the packet's first element
+        if (tFirst + 8 <= tLo || tFirst >= tHi) continue;
+        const T* src = sOut + j * outPitch + 8 * p;
+        T* dst = out + rowElem + tFirst;
+        if (tFirst >= tLo && tFirst + 8 <= tHi) {
+            *reinterpret_cast<u32x4*>(dst) = *reinterpret_cast<const u32x4*>(src);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (tFirst + e >= tLo && tFirst + e < tHi) dst[e] = src[e];
             }
         }
     }
@@ -343,15 +398,20 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     HS = envInt("DIOPI_ROCM_TOKATT_HS", HS);
     if (HS != 1 && HS != 2 && HS != 4) HS = 1;
     // tokens per work-group: with one query head per kv head, tiles of 64 tokens measured 1.7 % faster than 128 (64
-    // sequences of 512..2048 tokens, 32 heads); with 8 query heads per kv head 128 is 1.3 % faster than 64
-    int TT = envInt("DIOPI_ROCM_TOKATT_TT", a.G == 1 ? 64 : 128);
+    // sequences of 512..2048 tokens, 32 heads); with 8 query heads per kv head (128 sequences of 1024..8192 tokens, 8 kv
+    // heads) 256 is 4 % faster than 128 and 512 is 1 % slower than 256: longer pieces of every logits row per write-out
+    int TT = envInt("DIOPI_ROCM_TOKATT_TT", a.G == 1 ? 64 : 256);
     TT = TT / 64 * 64;
     if (TT < 64) TT = 64;
     if (TT > 1024) TT = 1024;
+    // the scores of a tile wait in LDS for the write-out: at most 40 KiB of them
+    const int outRows = HS * HW * a.G;
+    while (TT > 64 && outRows * (TT + 8) * static_cast<int>(sizeof(T)) > 40 * 1024) TT -= 64;
+    const size_t outLds = static_cast<size_t>(outRows) * (TT + 8) * sizeof(T);
     ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
     const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
 #define ROCM_STAGED_CASE(HWC)                                                                                                                         \
-    hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),                  \
+    hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), outLds, stream, static_cast<T*>(out), static_cast<const T*>(q),             \
                        static_cast<const T*>(k), a, TT, HS, scale)
     if (HW == 4) {
         ROCM_STAGED_CASE(4);

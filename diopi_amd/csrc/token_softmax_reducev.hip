@@ -97,7 +97,7 @@ __device__ __forceinline__ float waveSumUniform(float v) {
 }
 
 template <typename T, int GC, int HPW>
-__global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
+__global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
                                                                     SplitArgs sp) {
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
@@ -207,14 +207,22 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
         }
         waveLdsFence();
     };
-    u32x4 rowsV[8];
-    auto issueV = [&](int step) {
-        int32_t sidx[8];
+    // two sets of 8 rows per lane: while the products of one step consume a set, the rows of the next step are in flight
+    u32x4 rowsA[8], rowsB[8];
+    auto issueV = [&](int step, u32x4 (&rows)[8]) {
         const int first = HPW == 1 ? 32 * step + 8 * q : 8 * step;
-        *reinterpret_cast<u32x4*>(&sidx[0]) = *reinterpret_cast<const u32x4*>(slotW + first);
-        *reinterpret_cast<u32x4*>(&sidx[4]) = *reinterpret_cast<const u32x4*>(slotW + first + 4);
+        const u32x4 s0 = *reinterpret_cast<const u32x4*>(slotW + first);
+        const u32x4 s1 = *reinterpret_cast<const u32x4*>(slotW + first + 4);
 #pragma unroll
-        for (int r = 0; r < 8; ++r) rowsV[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(sidx[r]) * rowStride));
+        for (int r = 0; r < 4; ++r) {
+            rows[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(static_cast<int32_t>(s0[r])) * rowStride));
+            rows[4 + r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(static_cast<int32_t>(s1[r])) * rowStride));
+        }
+    };
+    constexpr int kStepsPerSub = kSub / kStep;  // even: a set keeps its parity from one sub-tile to the next
+    auto stepsOf = [&](int sub) {
+        const int n = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
+        return (n + kStep - 1) / kStep;
     };
 
     // the first logits are requested before the first rows: the softmax of sub-tile 0 then only waits for them, as
@@ -222,7 +230,8 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
     loadSlots(0);
     loadLogits(0);
     storeSlots();
-    issueV(0);
+    issueV(0, rowsA);
+    if (stepsOf(0) > 1) issueV(1, rowsB);
 
     f32x4 acc[8];
 #pragma unroll
@@ -270,9 +279,8 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
         // A operand: row c, the 8 tokens of this lane group's k slots; rows of other kv heads contribute zeros
         const bool rowLive = HPW == 1 ? c < G : (c < R && c / G == q);
         const T* pRow = tile + (c < R ? c : 0) * kTilePitch + (HPW == 1 ? 8 * q : 0);
-        // step 0 runs outside the loop: it waits for rows requested before the softmax and the prefetches above, the
-        // later steps for rows requested one step earlier; in one loop the compiler would make every step wait for all
-        auto pvStep = [&](int s) {
+        const int nStepsNext = (sub + 1 < nSub) ? stepsOf(sub + 1) : 0;
+        auto pvStep = [&](int s, u32x4 (&rowsV)[8]) {
             union {
                 u32x4 u;
                 Frag f;
@@ -294,16 +302,23 @@ __global__ __launch_bounds__(kRvThreads, 4) void softmaxReduceVWave(T* __restric
                 acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
                 acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
             }
-            // the row registers are free again: request the next rows (of this sub-tile or the first of the next one)
-            if (s + 1 < nSteps) {
-                issueV(s + 1);
-            } else if (sub + 1 < nSub) {
-                storeSlots();
-                issueV(0);
+            // this set of row registers is free again: request the rows two steps ahead (of this sub-tile or of the
+            // next one, whose slots take over the wave's LDS line once the last rows of this sub-tile are requested)
+            if (s + 2 < nSteps) {
+                issueV(s + 2, rowsV);
+            } else if (s + 2 - nSteps < nStepsNext) {
+                if (s + 2 == nSteps) storeSlots();
+                issueV(s + 2 - nSteps, rowsV);
             }
         };
-        pvStep(0);
-        for (int s = 1; s < nSteps; ++s) pvStep(s);
+        // the first two steps run outside the loop: they wait for rows requested before the softmax and the prefetches
+        // above, the later steps for rows requested two steps earlier
+        pvStep(0, rowsA);
+        if (nSteps > 1) pvStep(1, rowsB);
+        for (int s = 2; s < nSteps; s += 2) {
+            pvStep(s, rowsA);
+            if (s + 1 < nSteps) pvStep(s + 1, rowsB);
+        }
     }
 
     // ---- hand the denominators to the lanes that hold the matching accumulator rows, then store ----

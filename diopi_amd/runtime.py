@@ -21,7 +21,8 @@ from typing import Optional, Sequence
 
 import torch
 
-_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+# the in-tree build; DIOPI_AMD_LIB_DIR points the package at another build of the same two libraries
+_LIB_DIR = os.environ.get("DIOPI_AMD_LIB_DIR") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 RT_LIB_PATH = os.path.join(_LIB_DIR, "libdiopirt_hip.so")
 IMPL_LIB_PATH = os.path.join(_LIB_DIR, "libdiopi_impl.so")
 
