@@ -30,14 +30,24 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0    # dense fp16 / bf16
 WARM_SECONDS = 0.3          # untimed load before every timed region (clock ramp)
-# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one counter per run, commands
-# and raw readings in profiles/all_operators_cfg1-5_hbm_traffic.txt) for the seeded cfg3 workload, each counter scaled
-# by what it reads for a plain copy of known size (the 65536-row DestIndexCopyKV sweep: 1.9854 KiB per FETCH_SIZE
-# count, 1.0000 KiB per WRITE_SIZE count).  The counters cannot be read from inside this script.
-MEASURED_TRAFFIC_CFG3 = {
-    "tokenAttStaged": int((314021.0 * 1.9854 + 4996.9) * 1024),
-    "softmaxReduceVWave+Merge": int(((316226.9 + 1684.0) * 1.9854 + 2974.4 + 512.0) * 1024),
-}
+# HBM bytes per launch of the two decode kernels at the seeded cfg3 workload, measured with `rocprofv3 --pmc FETCH_SIZE`
+# and `--pmc WRITE_SIZE` (one counter per run).  The counters cannot be read from inside this script: the readings, the
+# scale of each counter (what it reads for a plain copy of known size) and the commands are kept in the file below,
+# which is rewritten whenever the decode kernels change; a line `<kernel> total_cached_tokens=<n> hbm_bytes=<b>` per kernel.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "decode_kernels_cfg3_hbm_traffic.txt")
+
+
+def measured_traffic(kernel, total_tokens):
+    """HBM bytes per launch of `kernel` from the tracked counter summary, or None when it has no line for this workload."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for ln in f:
+                parts = ln.split()
+                if len(parts) >= 3 and parts[0] == kernel and parts[1] == f"total_cached_tokens={total_tokens}" and parts[2].startswith("hbm_bytes="):
+                    return int(parts[2].split("=", 1)[1])
+    except OSError:
+        pass
+    return None
 
 
 def main():
@@ -71,13 +81,23 @@ def main():
     K, Wm = args.steps, args.warmup
     only = set(x for x in args.only.split(",") if x)
     cores = torch.get_num_threads()
+    # the first processor's identification as /proc/cpuinfo gives it: model name plus the numeric family / model / stepping
     cpu_model = "unknown"
     try:
+        ident = {}
         with open("/proc/cpuinfo") as f:
             for ln in f:
-                if ln.startswith("model name"):
-                    cpu_model = ln.split(":", 1)[1].strip()
-                    break
+                if ":" not in ln:
+                    if ident:
+                        break
+                    continue
+                key, val = (x.strip() for x in ln.split(":", 1))
+                if key in ("vendor_id", "model name", "cpu family", "model", "stepping", "cpu MHz"):
+                    ident[key] = val
+        if ident:
+            cpu_model = "{} ({}, family {} model {} stepping {}, {} MHz)".format(
+                ident.get("model name", "?"), ident.get("vendor_id", "?"), ident.get("cpu family", "?"), ident.get("model", "?"),
+                ident.get("stepping", "?"), ident.get("cpu MHz", "?"))
     except OSError:
         pass
 
@@ -318,29 +338,44 @@ def main():
         b_copy = 2 * W.destindex_bytes(B, Hkv, D, e)
         cpu = None
         if not args.no_cpu:
-            # bounded sample: the first sequences of the batch through the reference's per-sequence composition
+            # bounded sample: the first sequences of the batch through the reference's per-sequence composition; one
+            # untimed warm-up pass over the first sequence sizes the sample so that a warm-up pass and three timed
+            # passes over it fit the budget; the median of the three is reported
             qc, blc, bsc, bln = w["q"].cpu(), w["b_loc"].cpu(), w["b_start_loc"].cpu(), w["b_seq_len"].cpu()
-            nseq, spent, tok = 0, 0.0, 0
             budget = args.cpu_seconds if tag == "cfg3" else 4.0
-            while nseq < B and spent < budget:
-                sel = slice(nseq, nseq + 1)
+
+            def prepare(n):
+                sel = slice(n, n + 1)
                 used = torch.unique(blc[sel].long())
                 remap = torch.zeros(int(used.max()) + 1, dtype=torch.int32)
                 remap[used] = torch.arange(used.numel(), dtype=torch.int32)
-                ks, vs = w["k_cache"][used.to(dev)].cpu(), w["v_cache"][used.to(dev)].cpu()
-                loc = remap[blc[sel].long()]
-                lg = torch.zeros(H, total, dtype=w["dtype"])
-                oc = torch.zeros(1, H, D, dtype=w["dtype"])
+                return dict(sel=sel, ks=w["k_cache"][used.to(dev)].cpu(), vs=w["v_cache"][used.to(dev)].cpu(), loc=remap[blc[sel].long()],
+                            lg=torch.zeros(H, total, dtype=w["dtype"]), oc=torch.zeros(1, H, D, dtype=w["dtype"]))
+
+            def run(p):
                 t0 = time.perf_counter()
-                O.token_attention(qc[sel], ks, lg, loc, bsc[sel], bln[sel], mil)
-                O.token_softmax_reducev(lg, vs, oc, loc, bsc[sel], bln[sel], mil, 0)
-                spent += time.perf_counter() - t0
+                O.token_attention(qc[p["sel"]], p["ks"], p["lg"], p["loc"], bsc[p["sel"]], bln[p["sel"]], mil)
+                O.token_softmax_reducev(p["lg"], p["vs"], p["oc"], p["loc"], bsc[p["sel"]], bln[p["sel"]], mil, 0)
+                return time.perf_counter() - t0
+
+            first = prepare(0)
+            run(first)                      # warm-up: threads, allocator, code paths
+            per_tok = run(first) / max(1, int(bln[0]))
+            nseq, tok = 1, int(bln[0])
+            while nseq < B and per_tok * (tok + int(bln[nseq])) * 4 < budget:
                 tok += int(bln[nseq])
                 nseq += 1
+            sample = [first] + [prepare(n) for n in range(1, nseq)]
+            for p_ in sample[1:]:
+                run(p_)                     # warm-up pass over the rest of the sample
+            reps = sorted(sum(run(p_) for p_ in sample) for _ in range(3))
+            spent = reps[1]
             frac_tok = tok / total
-            cpu = dict(seconds_sample=round(spent, 3), sequences=nseq, tokens_per_s=round(nseq / spent, 2),
-                       GBs=round((b_att + b_red) * frac_tok / spent / 1e9, 3), cores=cores,
-                       sample=f"first {nseq} of {B} sequences ({tok} of {total} cached tokens), attention only, cache rows pre-gathered")
+            cpu = dict(seconds_sample=round(spent, 3), seconds_all_reps=[round(x, 3) for x in reps], sequences=nseq,
+                       tokens_per_s=round(nseq / spent, 2), GBs=round((b_att + b_red) * frac_tok / spent / 1e9, 3), cores=cores,
+                       sample=f"first {nseq} of {B} sequences ({tok} of {total} cached tokens), attention only, cache rows pre-gathered; "
+                              f"one warm-up pass, median of 3 timed passes")
+            del sample, first
         record("diopiDestIndexCopyKV x2 (K,V)", f"{tag} {B} tokens", ms_copy, b_copy, "hbm", dtype_name,
                note="launch-bound at this size: 1 MiB of traffic per call")
         record("diopiTokenAttentionInference", tag, ms_att, b_att, "hbm", dtype_name)
@@ -471,10 +506,11 @@ def main():
             kname, kms, kbytes = "tokenAttStaged (diopiTokenAttentionInference)", head["ms_att"], head["b_att"]
         else:
             kname, kms, kbytes = "softmaxReduceVWave+Merge (diopiTokenSoftmaxReduceVInference)", head["ms_red"], head["b_red"]
-        traffic = MEASURED_TRAFFIC_CFG3.get(kname.split(" ")[0]) if head["total"] == 78106 else None
+        traffic = measured_traffic(kname.split(" ")[0], head["total"])
         ach = kbytes / (kms * 1e-3) / 1e9
         line["roofline"] = {"bound": "hbm", "kernel": kname, "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5)}
+                            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic, "algorithmic_bytes": int(kbytes), "ms": round(kms, 5),
+                            "traffic_over_algorithmic": round(traffic / kbytes, 4) if traffic else None}
         if head["cpu"] is not None:
             c = head["cpu"]
             line["cpu_baseline"] = {"value": c["tokens_per_s"], "unit": "tokens/s", "cores": c["cores"], "kind": "port", "sample": c["sample"],

@@ -126,6 +126,27 @@ struct Mfma16<bf16_t> {
     static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 };
 
+// Reductions over the 16 lanes of a DPP row (quad permutes, then half-row and full-row mirrors); every lane of the
+// row ends with the result.  Four VALU moves instead of four trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dppMove(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float rowMax16(float v) {
+    v = fmaxf(v, dppMove<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dppMove<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dppMove<0x141>(v));  // row_half_mirror
+    v = fmaxf(v, dppMove<0x140>(v));  // row_mirror
+    return v;
+}
+__device__ __forceinline__ float rowSum16(float v) {
+    v += dppMove<0xB1>(v);
+    v += dppMove<0x4E>(v);
+    v += dppMove<0x141>(v);
+    v += dppMove<0x140>(v);
+    return v;
+}
+
 // Reads an index tensor element as int64 whatever its storage width.
 __device__ __forceinline__ int64_t loadIndex(const void* base, int64_t i, bool is64) {
     return is64 ? reinterpret_cast<const int64_t*>(base)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(base)[i]);

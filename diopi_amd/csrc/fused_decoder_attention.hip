@@ -1,0 +1,553 @@
+// diopiFusedDecoderAttentionInp for gfx950: one decode step of self-attention behind a single call, from the hidden
+// states to the attention output, over a contiguous per-sequence KV cache.
+//
+// Interface: proto/include/diopi/functions_lmdeploy.h:104-135 of the reference.  The reference holds the prototype and
+// five lines of prose, no implementation and no test; what the prose leaves open is decided here and listed below.
+// For batch row b that is not finished, with L = sequence_lengths[b] tokens already cached:
+//   1. qkv = T(inoutput[b, :] @ qkv_weight) + qkv_bias                  [(H + 2 Hkv) * D], fp32 accumulate
+//   2. q and k heads rotate at position step - 1 - total_padding_tokens[b] with the half-split pairing of
+//      diopiRotaryEmbedding (dims j and j + D/2, angle pos * rope_theta^(-2j/D)); the sums of 1 and the rotation are
+//      done in fp32 and rounded once to the element type
+//   3. k and v go to key_cache / value_cache [layer_id, b, kv head, L % max_seq_len, :]
+//   4. out[b, h, :] = sum_j p_j v_j over the last min(L + 1, max_seq_len) cached tokens (the new one included),
+//      p_j = exp(s_j - max s) / (sum exp(s - max s) + 1e-6), s_j = (q_h . k_j) / sqrt(D), query head h reading kv head
+//      h / (H / Hkv); fp32 scores and sums, probabilities rounded to the element type before the product with V
+//   5. inoutput[b, 0 : H*D] = out[b] (H*D <= hidden_units; columns past H*D keep their values)
+// Open in the prose, fixed here: the rotary pairing (2), a circular cache window once L reaches max_seq_len (3, 4),
+// where the output lands when H*D < hidden_units (5), and that finished rows are left untouched everywhere.
+//
+// Three kernels, all on the context's stream:
+//   fusedQkvHead     one work-group per head of the projection (128 output columns) and 64 batch rows.  The weight
+//                    panel [hidden, 128] is streamed once: 8 waves = 4 row blocks of 16 batch rows x 2 halves of the
+//                    hidden dimension.  A lane loads 8 consecutive weight rows (16 bytes = 8 columns each); pairs of rows
+//                    interleaved with two byte permutes become the B operands of v_mfma_f32_16x16x32 for the lane's 8
+//                    columns, the A operand is 16 bytes of a hidden-state row.  The two halves meet in LDS (fp32), and
+//                    the same work-group adds the bias, rotates, and writes the head: q to the workspace, k and v
+//                    straight into the cache.  HBM-bound on the weights.
+//   fusedDecodeAttn  a wave owns (batch row, kv head, range of cached tokens): per 32 tokens 8 K loads that arrive in
+//                    the B-operand layout of q.k^T (16 lanes x 16-byte pieces of 16 consecutive cache rows), online
+//                    softmax on the 16 x 32 scores (row maxima and sums by DPP row reductions), probabilities through a
+//                    wave-private LDS tile into the A-operand layout, 8 V loads permuted as above for P.V.  The scores
+//                    never leave the chip: per cached token the kernel reads its K row and its V row and nothing else.
+//   fusedDecodeMerge combines the ranges of a row (skipped when the window fits one range).
+#include <diopi/functions_lmdeploy.h>
+
+#include <cmath>
+
+#include "common.hpp"
+#include "device.hpp"
+
+namespace rocm {
+namespace {
+
+constexpr int kFD = 128;          // head size of the fast path
+constexpr int kProjThreads = 512;
+constexpr int kProjSlabs = kProjThreads / kWave / 4;  // slabs of the hidden dimension: waves = 4 row blocks x slabs
+constexpr int kProjRows = 64;     // batch rows per work-group of the projection
+constexpr int kProjPitch = kFD + 4;  // floats per row of a partial tile: rows 4 apart are 16 banks apart
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / kWave;
+constexpr int kAttnStep = 32;     // cached tokens per step of a wave
+constexpr int kProbPitch = kAttnStep + 8;  // elements per row of the probability tile
+
+struct FusedArgs {
+    const void* finished;  // [B] one byte per row, or null
+    const void* padding;   // [B] total_padding_tokens, or null
+    const void* seqLen;    // [B] sequence_lengths
+    bool pad64, len64;
+    int B, hidden, H, Hkv, G;
+    int64_t step;
+    int maxSeq;
+    int rot;               // rotating dims of a head: 0 or kFD
+    float ropeTheta;
+    int64_t layerOffset;   // elements from the start of a cache to the layer's [B, Hkv, maxSeq, D] block
+};
+
+__device__ __forceinline__ bool rowFinished(const FusedArgs& a, int b) {
+    return a.finished != nullptr && reinterpret_cast<const unsigned char*>(a.finished)[b] != 0;
+}
+__device__ __forceinline__ int64_t rowLength(const FusedArgs& a, int b) {
+    const int64_t L = loadIndex(a.seqLen, b, a.len64);
+    return L < 0 ? 0 : L;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const T* __restrict__ x,
+                                                            const T* __restrict__ w, const T* __restrict__ bias, FusedArgs a) {
+    using Ops = Mfma16<T>;
+    using Frag = typename Ops::Frag;
+    extern __shared__ __attribute__((aligned(16))) float part[];  // [kProjSlabs][64 rows][kProjPitch]
+    const int tile = blockIdx.x;  // head of the projection: H query heads, then Hkv key heads, then Hkv value heads
+    const int rowBase = blockIdx.y * kProjRows;
+    const int N = (a.H + 2 * a.Hkv) * kFD;
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int rb = wave % 4;   // block of 16 batch rows
+    const int ks = wave / 4;   // slab of the hidden dimension
+    const int g4 = lane / 16;  // A, B: k slots 8 g4 .. + 7 of a 32-row step; C: rows 4 g4 .. + 3
+    const int c = lane % 16;   // A: batch row of the block; loads: 16-byte packet (8 columns) of the panel; C: column
+    const int kPer = a.hidden / kProjSlabs;  // a multiple of 32
+    const int steps = kPer / 32;
+    int row = rowBase + rb * 16 + c;
+    row = row < a.B ? row : a.B - 1;
+    const T* xRow = x + static_cast<int64_t>(row) * a.hidden + ks * kPer + 8 * g4;
+    const T* wCol = w + static_cast<int64_t>(ks * kPer + 8 * g4) * N + tile * kFD + 8 * c;
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    struct Step {
+        u32x4 w[8];
+        u32x4 x;
+    };
+    // every step issues the same loads (past the last step the last one again), so that the wait for one step's rows
+    // leaves exactly the next step's in flight
+    auto issue = [&](int s, Step& st) {
+        const int sc = s < steps ? s : steps - 1;
+        st.x = *reinterpret_cast<const u32x4*>(xRow + 32 * sc);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) st.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wCol + static_cast<int64_t>(32 * sc + r) * N));
+    };
+    auto consume = [&](const Step& st) {
+        union {
+            u32x4 u;
+            Frag f;
+        } pa;
+        pa.u = st.x;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            union {
+                u32x4 u;
+                Frag f;
+            } lo, hi;
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {
+                // columns 2j and 2j+1 of this lane's packet, weight rows (2pr, 2pr+1) of the lane group
+                lo.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x05040100u);
+                hi.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x07060302u);
+            }
+            acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
+            acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
+        }
+    };
+    Step sa, sb;
+    issue(0, sa);
+    issue(1, sb);
+    for (int s = 0; s < steps; s += 2) {
+        consume(sa);
+        issue(s + 2, sa);
+        if (s + 1 < steps) consume(sb);
+        issue(s + 3, sb);
+    }
+    // acc[e][r] is the sum of this slab for batch row rb*16 + 4 g4 + r, column 8c + e
+    float* mine = part + (ks * kProjRows + rb * 16 + 4 * g4) * kProjPitch + 8 * c;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        *reinterpret_cast<f32x4*>(mine + r * kProjPitch) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        *reinterpret_cast<f32x4*>(mine + r * kProjPitch + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+    }
+    __syncthreads();
+
+    // ---- bias, rotation, and the head's destination: a thread takes the pair (j, j + 64) of a batch row
+    const bool isQ = tile < a.H;
+    const bool isK = !isQ && tile < a.H + a.Hkv;
+    const int head = isQ ? tile : (isK ? tile - a.H : tile - a.H - a.Hkv);
+    for (int idx = threadIdx.x; idx < kProjRows * (kFD / 2); idx += kProjThreads) {
+        const int r = idx / (kFD / 2);
+        const int j = idx % (kFD / 2);
+        const int b = rowBase + r;
+        if (b >= a.B || rowFinished(a, b)) continue;
+        float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+        for (int k4 = 0; k4 < kProjSlabs; ++k4) {
+            v0 += part[(k4 * kProjRows + r) * kProjPitch + j];
+            v1 += part[(k4 * kProjRows + r) * kProjPitch + j + kFD / 2];
+        }
+        // the product is rounded to the element type as a matrix product in that type would leave it
+        float y0 = toFloat(fromFloat<T>(v0)), y1 = toFloat(fromFloat<T>(v1));
+        if (bias != nullptr) {
+            y0 += toFloat(bias[tile * kFD + j]);
+            y1 += toFloat(bias[tile * kFD + j + kFD / 2]);
+        }
+        if ((isQ || isK) && a.rot > 0) {
+            const int64_t pad = a.padding != nullptr ? loadIndex(a.padding, b, a.pad64) : 0;
+            const float pos = static_cast<float>(a.step - 1 - pad);
+            const float invFreq = exp2f(-(2.0f * static_cast<float>(j) / static_cast<float>(a.rot)) * log2f(a.ropeTheta));
+            float sn, cs;
+            sincosf(pos * invFreq, &sn, &cs);
+            const float o0 = y0 * cs - y1 * sn;
+            const float o1 = y0 * sn + y1 * cs;
+            y0 = o0;
+            y1 = o1;
+        }
+        T* dst;
+        if (isQ) {
+            dst = qOut + (static_cast<int64_t>(b) * a.H + head) * kFD;
+        } else {
+            const int64_t slot = rowLength(a, b) % a.maxSeq;
+            dst = (isK ? kCache : vCache) + a.layerOffset + ((static_cast<int64_t>(b) * a.Hkv + head) * a.maxSeq + slot) * kFD;
+        }
+        dst[j] = fromFloat<T>(y0);
+        dst[j + kFD / 2] = fromFloat<T>(y1);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+struct AttnSplit {
+    float* partAcc;  // [B, splits, H, D]
+    float* partMl;   // [B, splits, H, 2]  (maximum, denominator)
+    int splits;      // ranges per row the workspace is sized for
+    int TT;          // cached tokens per range (a multiple of kAttnStep)
+};
+
+template <typename T>
+__global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict__ out, const T* __restrict__ qIn, const T* __restrict__ kCache,
+                                                                   const T* __restrict__ vCache, FusedArgs a, AttnSplit sp) {
+    using Ops = Mfma16<T>;
+    using Frag = typename Ops::Frag;
+    __shared__ __attribute__((aligned(16))) T sP[kAttnWaves][16 * kProbPitch];
+    const int b = blockIdx.y;
+    const int split = blockIdx.z;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int hk = blockIdx.x * kAttnWaves + wave;
+    if (hk >= a.Hkv || rowFinished(a, b)) return;  // waves never meet at a barrier
+    const int64_t L = rowLength(a, b);
+    const int nWin = static_cast<int>(L + 1 < a.maxSeq ? L + 1 : a.maxSeq);  // tokens in the window, the new one last
+    const int t0 = split * sp.TT;
+    if (t0 >= nWin) return;
+    const int nTok = nWin - t0 < sp.TT ? nWin - t0 : sp.TT;
+    const int nSteps = (nTok + kAttnStep - 1) / kAttnStep;
+    const int firstPos = static_cast<int>((L + 1 - nWin) % a.maxSeq);  // cache row of the window's first token
+    const int g4 = lane / 16;
+    const int c = lane % 16;
+    const int G = a.G;
+    const int64_t headOff = a.layerOffset + (static_cast<int64_t>(b) * a.Hkv + hk) * a.maxSeq * kFD;
+    const T* kHead = kCache + headOff + 8 * g4;  // + row * D + 32 s: 8 dims of k block g4
+    const T* vHead = vCache + headOff + 8 * c;   // + row * D: packet c of a row
+    T* tile = sP[wave];
+    // cache row of token i of the range; tokens past the range repeat its last one (their scores become -inf)
+    auto rowOf = [&](int i) {
+        int p = firstPos + t0 + (i < nTok ? i : nTok - 1);
+        p = p >= a.maxSeq ? p - a.maxSeq : p;
+        return static_cast<int64_t>(p) * kFD;
+    };
+    // A fragments of q.k^T: row c is query head hk*G + c (zero beyond the group)
+    Frag qa[kFD / 32];
+#pragma unroll
+    for (int s = 0; s < kFD / 32; ++s) {
+        union {
+            u32x4 raw;
+            Frag f;
+        } u;
+        u.raw = u32x4{0u, 0u, 0u, 0u};
+        if (c < G) u.raw = *reinterpret_cast<const u32x4*>(qIn + (static_cast<int64_t>(b) * a.H + hk * G + c) * kFD + 32 * s + 8 * g4);
+        qa[s] = u.f;
+    }
+    u32x4 kb[2][kFD / 32], vb[8];
+    auto issueK = [&](int st) {
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+            const T* p = kHead + rowOf(kAttnStep * st + 16 * tg + c);
+#pragma unroll
+            for (int s = 0; s < kFD / 32; ++s) kb[tg][s] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + 32 * s));
+        }
+    };
+    auto issueV = [&](int st) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) vb[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + rowOf(kAttnStep * st + 8 * g4 + r)));
+    };
+    issueK(0);
+    issueV(0);
+
+    f32x4 acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mRun[4], lRun[4];  // of query heads 4 g4 + r (the same in the 16 lanes of a row group)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        mRun[r] = -INFINITY;
+        lRun[r] = 0.f;
+    }
+    const float scale = 1.0f / sqrtf(static_cast<float>(kFD));
+    const bool rowLive = c < G;
+
+    for (int st = 0; st < nSteps; ++st) {
+        // ---- scores of 32 tokens: C holds query heads 4 g4 + r of token column c of each 16-token group
+        f32x4 sc[2];
+#pragma unroll
+        for (int tg = 0; tg < 2; ++tg) {
+            sc[tg] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < kFD / 32; ++s) {
+                union {
+                    u32x4 raw;
+                    Frag f;
+                } u;
+                u.raw = kb[tg][s];
+                sc[tg] = Ops::mma(qa[s], u.f, sc[tg]);
+            }
+        }
+        issueK(st + 1);  // the K registers are free: the next step's rows (past the range: its last row again)
+        float alpha[4];
+        bool moved = false;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool ok0 = kAttnStep * st + c < nTok, ok1 = kAttnStep * st + 16 + c < nTok;
+            const float s0 = ok0 ? sc[0][r] * scale : -INFINITY;
+            const float s1 = ok1 ? sc[1][r] * scale : -INFINITY;
+            const float mNew = fmaxf(mRun[r], rowMax16(fmaxf(s0, s1)));  // finite: every step holds a token of the range
+            const float p0 = __expf(s0 - mNew), p1 = __expf(s1 - mNew);
+            alpha[r] = __expf(mRun[r] - mNew);  // 0 on the first step
+            moved = moved || mNew != mRun[r];
+            lRun[r] = lRun[r] * alpha[r] + rowSum16(p0 + p1);
+            mRun[r] = mNew;
+            tile[(4 * g4 + r) * kProbPitch + c] = static_cast<T>(p0);
+            tile[(4 * g4 + r) * kProbPitch + 16 + c] = static_cast<T>(p1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        if (__any(moved)) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[e][r] *= alpha[r];
+            }
+        }
+        // ---- P . V: A operand row c, tokens 8 g4 .. + 7; B operands from the lane's 8 V rows
+        union {
+            u32x4 u;
+            Frag f;
+        } pa;
+        pa.u = *reinterpret_cast<const u32x4*>(tile + c * kProbPitch + 8 * g4);
+        if (!rowLive) pa.u = u32x4{0u, 0u, 0u, 0u};
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            union {
+                u32x4 u;
+                Frag f;
+            } lo, hi;
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr) {
+                lo.u[pr] = __builtin_amdgcn_perm(vb[2 * pr + 1][j], vb[2 * pr][j], 0x05040100u);
+                hi.u[pr] = __builtin_amdgcn_perm(vb[2 * pr + 1][j], vb[2 * pr][j], 0x07060302u);
+            }
+            acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
+            acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
+        }
+        issueV(st + 1);
+    }
+
+    // ---- acc[e][r] is dim 8c + e of query head 4 g4 + r
+    const bool single = nWin <= sp.TT;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int g = 4 * g4 + r;
+        if (g >= G) continue;
+        const int qh = hk * G + g;
+        if (single) {
+            const float inv = 1.0f / (lRun[r] + 1e-6f);
+            Pack16<T> o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.e[e] = static_cast<T>(acc[e][r] * inv);
+            storePack(out + static_cast<int64_t>(b) * a.hidden + qh * kFD + 8 * c, o);
+        } else {
+            const int64_t slot = (static_cast<int64_t>(b) * sp.splits + split) * a.H + qh;
+            float* dst = sp.partAcc + slot * kFD + 8 * c;
+            *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+            if (c == 0) {
+                sp.partMl[slot * 2] = mRun[r];
+                sp.partMl[slot * 2 + 1] = lRun[r];
+            }
+        }
+    }
+}
+
+// out[b, h, :] = sum_j w_j acc_j / (sum_j w_j l_j + 1e-6), w_j = exp(m_j - max m), over the ranges of row b
+template <typename T>
+__global__ __launch_bounds__(256) void fusedDecodeMerge(T* __restrict__ out, FusedArgs a, AttnSplit sp) {
+    const int b = blockIdx.y;
+    if (rowFinished(a, b)) return;
+    const int64_t L = rowLength(a, b);
+    const int nWin = static_cast<int>(L + 1 < a.maxSeq ? L + 1 : a.maxSeq);
+    if (nWin <= sp.TT) return;  // finished by the attention kernel
+    const int ns = (nWin + sp.TT - 1) / sp.TT;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= a.H * kFD) return;
+    const int qh = idx / kFD, d = idx % kFD;
+    const float* ml = sp.partMl + (static_cast<int64_t>(b) * sp.splits * a.H + qh) * 2;
+    const float* pa = sp.partAcc + (static_cast<int64_t>(b) * sp.splits * a.H + qh) * kFD + d;
+    float m = -INFINITY;
+    for (int j = 0; j < ns; ++j) m = fmaxf(m, ml[static_cast<int64_t>(j) * a.H * 2]);
+    float num = 0.f, den = 0.f;
+    for (int j = 0; j < ns; ++j) {
+        const float wgt = __expf(ml[static_cast<int64_t>(j) * a.H * 2] - m);
+        num += wgt * pa[static_cast<int64_t>(j) * a.H * kFD];
+        den += wgt * ml[static_cast<int64_t>(j) * a.H * 2 + 1];
+    }
+    out[static_cast<int64_t>(b) * a.hidden + idx] = static_cast<T>(num / (den + 1e-6f));
+}
+
+template <typename T>
+diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const void* bias, void* workspace, void* kCache, void* vCache, const FusedArgs& a,
+                         const AttnSplit& spIn, int64_t qBytes) {
+    T* qBuf = static_cast<T*>(workspace);
+    AttnSplit sp = spIn;
+    sp.partAcc = reinterpret_cast<float*>(static_cast<char*>(workspace) + qBytes);
+    sp.partMl = sp.partAcc + static_cast<int64_t>(a.B) * sp.splits * a.H * kFD;
+    const size_t projLds = static_cast<size_t>(kProjSlabs) * kProjRows * kProjPitch * sizeof(float);
+    ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(fusedQkvHead<T>), static_cast<int>(projLds)));
+    const dim3 pgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, kProjRows)));
+    hipLaunchKernelGGL((fusedQkvHead<T>), pgrid, dim3(kProjThreads), projLds, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache),
+                       static_cast<const T*>(inout), static_cast<const T*>(w), static_cast<const T*>(bias), a);
+    ROCM_LAUNCH_CHECK();
+    const dim3 agrid(static_cast<unsigned>(ceilDiv(a.Hkv, kAttnWaves)), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
+    hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), 0, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
+                       static_cast<const T*>(vCache), a, sp);
+    ROCM_LAUNCH_CHECK();
+    if (sp.splits > 1) {
+        const dim3 mgrid(static_cast<unsigned>(ceilDiv(static_cast<int64_t>(a.H) * kFD, 256)), static_cast<unsigned>(a.B));
+        hipLaunchKernelGGL((fusedDecodeMerge<T>), mgrid, dim3(256), 0, stream, static_cast<T*>(inout), a, sp);
+        ROCM_LAUNCH_CHECK();
+    }
+    return diopiSuccess;
+}
+
+diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t inoutput, diopiConstTensorHandle_t qkv_weight, diopiConstTensorHandle_t qkv_bias,
+                                   diopiTensorHandle_t workspace, int64_t* workspace_size, int64_t fusion_level, diopiTensorHandle_t key_cache,
+                                   diopiTensorHandle_t value_cache, diopiConstTensorHandle_t finished, diopiConstTensorHandle_t total_padding_tokens,
+                                   diopiConstTensorHandle_t sequence_lengths, int64_t step, int64_t layer_id, int64_t local_head_num,
+                                   int64_t local_kv_head_num, int64_t size_per_head, int64_t max_seq_len, int64_t rotary_embedding, float rope_theta) {
+    (void)fusion_level;  // every level gets the same three kernels
+    TensorView vX, vW, vB, vWs, vK, vV, vF, vP, vL;
+    ROCM_CALL(unwrap(inoutput, "inoutput", &vX));
+    ROCM_CALL(unwrap(qkv_weight, "qkv_weight", &vW));
+    ROCM_CALL(unwrap(key_cache, "key_cache", &vK));
+    ROCM_CALL(unwrap(value_cache, "value_cache", &vV));
+    ROCM_CALL(unwrap(sequence_lengths, "sequence_lengths", &vL));
+    ROCM_CALL(requireDeviceContiguous(vX, "inoutput"));
+    ROCM_CALL(requireDeviceContiguous(vW, "qkv_weight"));
+    ROCM_CALL(requireDeviceContiguous(vK, "key_cache"));
+    ROCM_CALL(requireDeviceContiguous(vV, "value_cache"));
+    ROCM_CALL(requireDeviceContiguous(vL, "sequence_lengths"));
+    ROCM_CHECK(workspace_size != nullptr, "workspace_size must not be null");
+    ROCM_CHECK(vX.ndim == 2, "inoutput must be [batch_size, hidden_units]");
+    const int64_t B = vX.shape[0], hidden = vX.shape[1];
+    const int64_t H = local_head_num, Hkv = local_kv_head_num, D = size_per_head;
+    ROCM_CHECK(H > 0 && Hkv > 0 && H % Hkv == 0, "local_head_num %lld must be a positive multiple of local_kv_head_num %lld", static_cast<long long>(H),
+               static_cast<long long>(Hkv));
+    const int64_t N = (H + 2 * Hkv) * D;
+    ROCM_CHECK(vW.ndim == 2 && vW.shape[0] == hidden && vW.shape[1] == N && vW.dtype == vX.dtype,
+               "qkv_weight must be [hidden_units, (local_head_num + 2 local_kv_head_num) size_per_head] = [%lld, %lld] of dtype %s",
+               static_cast<long long>(hidden), static_cast<long long>(N), dtypeName(vX.dtype));
+    ROCM_CHECK(H * D <= hidden, "the attention output [local_head_num * size_per_head = %lld] does not fit hidden_units = %lld", static_cast<long long>(H * D),
+               static_cast<long long>(hidden));
+    ROCM_CHECK(max_seq_len > 0 && max_seq_len < (int64_t(1) << 31) / D, "max_seq_len %lld is out of range", static_cast<long long>(max_seq_len));
+    ROCM_CHECK(vK.ndim == 5 && vK.shape[1] == B && vK.shape[2] == Hkv && vK.shape[3] == max_seq_len && vK.shape[4] == D && vK.dtype == vX.dtype,
+               "key_cache must be [num_layer, batch, local_kv_head_num, max_seq_len, size_per_head] of dtype %s", dtypeName(vX.dtype));
+    ROCM_CHECK(vV.sameShape(vK) && vV.dtype == vK.dtype, "value_cache must have the shape and dtype of key_cache");
+    ROCM_CHECK(layer_id >= 0 && layer_id < vK.shape[0], "layer_id %lld is outside the %lld layers of the caches", static_cast<long long>(layer_id),
+               static_cast<long long>(vK.shape[0]));
+    ROCM_CHECK(isIndexDtype(vL.dtype) && vL.numel == B, "sequence_lengths must hold batch_size = %lld int32 or int64 values", static_cast<long long>(B));
+    const void* biasPtr = nullptr;
+    if (qkv_bias != nullptr) {
+        ROCM_CALL(unwrap(qkv_bias, "qkv_bias", &vB));
+        ROCM_CALL(requireDeviceContiguous(vB, "qkv_bias"));
+        ROCM_CHECK(vB.numel == N && vB.dtype == vX.dtype, "qkv_bias must hold %lld elements of dtype %s", static_cast<long long>(N), dtypeName(vX.dtype));
+        biasPtr = vB.data;
+    }
+    FusedArgs a;
+    a.finished = nullptr;
+    if (finished != nullptr) {
+        ROCM_CALL(unwrap(finished, "finished", &vF));
+        ROCM_CALL(requireDeviceContiguous(vF, "finished"));
+        ROCM_CHECK(vF.numel == B && vF.itemsize() == 1, "finished must hold batch_size = %lld one-byte values", static_cast<long long>(B));
+        a.finished = vF.data;
+    }
+    a.padding = nullptr;
+    a.pad64 = false;
+    if (total_padding_tokens != nullptr) {
+        ROCM_CALL(unwrap(total_padding_tokens, "total_padding_tokens", &vP));
+        ROCM_CALL(requireDeviceContiguous(vP, "total_padding_tokens"));
+        ROCM_CHECK(isIndexDtype(vP.dtype) && vP.numel == B, "total_padding_tokens must hold batch_size = %lld int32 or int64 values", static_cast<long long>(B));
+        a.padding = vP.data;
+        a.pad64 = vP.dtype == diopi_dtype_int64;
+    }
+    // what this build implements: 16-bit elements, heads of 128, up to 16 query heads per kv head, rotation of the whole head
+    // or none, a hidden size the projection's slabs of 32-row steps divide, 16-byte aligned rows
+    const bool supported = (vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16) && D == kFD && H / Hkv <= 16 &&
+                           (rotary_embedding == 0 || rotary_embedding == kFD) && hidden % 128 == 0 && hidden >= 256 &&
+                           ((reinterpret_cast<uintptr_t>(vX.data) | reinterpret_cast<uintptr_t>(vW.data) | reinterpret_cast<uintptr_t>(vK.data) |
+                             reinterpret_cast<uintptr_t>(vV.data)) & 15) == 0;
+    if (!supported) {
+        setLastError("diopiFusedDecoderAttentionInp: only float16 / bfloat16, size_per_head 128, at most 16 query heads per kv head, rotary_embedding 0 or "
+                     "128 and hidden_units a multiple of 128 are implemented (got %s, %lld, %lld, %lld, %lld)",
+                     dtypeName(vX.dtype), static_cast<long long>(D), static_cast<long long>(H / Hkv), static_cast<long long>(rotary_embedding),
+                     static_cast<long long>(hidden));
+        return diopiNoImplement;
+    }
+    // ranges of the attention kernel: 256 cached tokens each when kv heads are plentiful, the workspace sized for max_seq_len
+    AttnSplit sp;
+    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 256);
+    sp.TT = static_cast<int>(ceilDiv(sp.TT, kAttnStep)) * kAttnStep;
+    sp.splits = static_cast<int>(ceilDiv(max_seq_len, sp.TT));
+    sp.partAcc = nullptr;
+    sp.partMl = nullptr;
+    ROCM_CHECK(B <= 65535 && sp.splits <= 65535, "batch %lld / max_seq_len %lld exceed the launch limits", static_cast<long long>(B),
+               static_cast<long long>(max_seq_len));
+    const int64_t e = vX.itemsize();
+    const int64_t qBytes = ceilDiv(B * H * D * e, 256) * 256;
+    const int64_t partBytes = sp.splits > 1 ? B * sp.splits * H * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
+    const int64_t need = qBytes + partBytes;
+    if (*workspace_size < 0) {
+        *workspace_size = need;  // size query: nothing else happens
+        return diopiSuccess;
+    }
+    void* wsPtr = nullptr;
+    if (workspace != nullptr) {
+        ROCM_CALL(unwrap(workspace, "workspace", &vWs));
+        ROCM_CALL(requireDeviceContiguous(vWs, "workspace"));
+        ROCM_CHECK(vWs.nbytes() >= need && *workspace_size >= need, "workspace holds %lld bytes (workspace_size %lld), %lld are needed",
+                   static_cast<long long>(vWs.nbytes()), static_cast<long long>(*workspace_size), static_cast<long long>(need));
+        ROCM_CHECK((reinterpret_cast<uintptr_t>(vWs.data) & 15) == 0, "workspace must be 16-byte aligned");
+        wsPtr = vWs.data;
+    } else {
+        ROCM_CALL(requireScratch(ctx, need, &wsPtr));  // a caller without a workspace tensor gets context scratch
+    }
+    if (B == 0) return diopiSuccess;
+    a.seqLen = vL.data;
+    a.len64 = vL.dtype == diopi_dtype_int64;
+    a.B = static_cast<int>(B);
+    a.hidden = static_cast<int>(hidden);
+    a.H = static_cast<int>(H);
+    a.Hkv = static_cast<int>(Hkv);
+    a.G = static_cast<int>(H / Hkv);
+    a.step = step;
+    a.maxSeq = static_cast<int>(max_seq_len);
+    a.rot = static_cast<int>(rotary_embedding);
+    a.ropeTheta = rope_theta;
+    a.layerOffset = layer_id * B * Hkv * max_seq_len * D;
+    hipStream_t stream;
+    ROCM_CALL(getStream(ctx, &stream));
+    if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes);
+    return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes);
+}
+
+}  // namespace
+}  // namespace rocm
+
+extern "C" diopiError_t diopiFusedDecoderAttentionInp(diopiContextHandle_t ctx, diopiTensorHandle_t inoutput, diopiConstTensorHandle_t qkv_weight,
+                                                      diopiConstTensorHandle_t qkv_bias, diopiTensorHandle_t workspace, int64_t* workspace_size,
+                                                      int64_t fusion_level, diopiTensorHandle_t key_cache, diopiTensorHandle_t value_cache,
+                                                      diopiConstTensorHandle_t finished, diopiConstTensorHandle_t total_padding_tokens,
+                                                      diopiConstTensorHandle_t sequence_lengths, int64_t step, int64_t layer_id, int64_t local_head_num,
+                                                      int64_t local_kv_head_num, int64_t size_per_head, int64_t max_seq_len, int64_t rotary_embedding,
+                                                      float rope_theta) {
+    ROCM_ENTRY_BEGIN
+    return rocm::fusedDecoderAttention(ctx, inoutput, qkv_weight, qkv_bias, workspace, workspace_size, fusion_level, key_cache, value_cache, finished,
+                                       total_padding_tokens, sequence_lengths, step, layer_id, local_head_num, local_kv_head_num, size_per_head, max_seq_len,
+                                       rotary_embedding, rope_theta);
+    ROCM_ENTRY_END
+}

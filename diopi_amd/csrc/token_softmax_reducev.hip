@@ -28,27 +28,6 @@ constexpr int kRvWaves = kRvThreads / kWave;
 constexpr int kSub = 128;          // tokens per sub-tile
 constexpr int kD = 128;
 
-// Reductions over the 16 lanes of a DPP row (quad permutes, then half-row and full-row mirrors); every lane of the
-// row ends with the result.  Four VALU moves instead of four trips through the LDS crossbar.
-template <int CTRL>
-__device__ __forceinline__ float dppMove(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float rowMax16(float v) {
-    v = fmaxf(v, dppMove<0xB1>(v));   // quad_perm [1,0,3,2]
-    v = fmaxf(v, dppMove<0x4E>(v));   // quad_perm [2,3,0,1]
-    v = fmaxf(v, dppMove<0x141>(v));  // row_half_mirror
-    v = fmaxf(v, dppMove<0x140>(v));  // row_mirror
-    return v;
-}
-__device__ __forceinline__ float rowSum16(float v) {
-    v += dppMove<0xB1>(v);
-    v += dppMove<0x4E>(v);
-    v += dppMove<0x141>(v);
-    v += dppMove<0x140>(v);
-    return v;
-}
-
 struct SplitArgs {
     float* partAcc;  // [batch, splits, H, D]
     float* partMl;   // [batch, splits, H, 2]  (running max, denominator)
@@ -219,7 +198,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
             rows[4 + r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(static_cast<int32_t>(s1[r])) * rowStride));
         }
     };
-    constexpr int kStepsPerSub = kSub / kStep;  // even: a set keeps its parity from one sub-tile to the next
+    static_assert((kSub / kStep) % 2 == 0, "a set of row registers keeps its parity from one sub-tile to the next");
     auto stepsOf = [&](int sub) {
         const int n = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
         return (n + kStep - 1) / kStep;

@@ -19,6 +19,8 @@ from typing import Optional, Sequence
 
 import math
 
+import ctypes
+
 import torch
 
 from . import runtime as rt
@@ -160,6 +162,32 @@ def fused_add_root_mean_square_norm_inp(inoutput: torch.Tensor, residual: torch.
         ret = rt.libs().impl.diopiFusedAddRootMeanSquareNormInp(ctx.handle, h[0], h[1], h[2], h[3], float(eps))
     check_returncode(ret, "diopiFusedAddRootMeanSquareNormInp")
     return inoutput, residual
+
+
+def fused_decoder_attention_inp(inoutput: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: Optional[torch.Tensor], workspace: Optional[torch.Tensor],
+                                fusion_level: int, key_cache: torch.Tensor, value_cache: torch.Tensor, finished: Optional[torch.Tensor],
+                                total_padding_tokens: Optional[torch.Tensor], sequence_lengths: torch.Tensor, step: int, layer_id: int, local_head_num: int,
+                                local_kv_head_num: int, size_per_head: int, max_seq_len: int, rotary_embedding: int, rope_theta: float,
+                                ctx: Optional[rt.Context] = None) -> torch.Tensor:
+    """One decode step of self-attention, from hidden states to attention output (functions_lmdeploy.h:104-135 of the reference).
+
+    `workspace` None allocates one of the size the operator asks for (the header's size query: workspace_size < 0)."""
+    ctx = _ctx(ctx)
+    with _on_stream(ctx, inoutput):
+        keep, h = _handles(inoutput, qkv_weight, qkv_bias, key_cache, value_cache, finished, total_padding_tokens, sequence_lengths)
+        args = (int(fusion_level), h[3], h[4], h[5], h[6], h[7], int(step), int(layer_id), int(local_head_num), int(local_kv_head_num), int(size_per_head),
+                int(max_seq_len), int(rotary_embedding), float(rope_theta))
+        if workspace is None:
+            size = ctypes.c_int64(-1)
+            ret = rt.libs().impl.diopiFusedDecoderAttentionInp(ctx.handle, h[0], h[1], h[2], None, ctypes.byref(size), *args)
+            check_returncode(ret, "diopiFusedDecoderAttentionInp (size query)")
+            workspace = torch.empty(max(int(size.value), 16), dtype=torch.int8, device=inoutput.device)
+        size = ctypes.c_int64(workspace.numel() * workspace.element_size())
+        keep_ws, hw = _handles(workspace)
+        ret = rt.libs().impl.diopiFusedDecoderAttentionInp(ctx.handle, h[0], h[1], h[2], hw[0], ctypes.byref(size), *args)
+    check_returncode(ret, "diopiFusedDecoderAttentionInp")
+    ctx.clear_tensors()
+    return inoutput
 
 
 def destindex_copy_kv(k: torch.Tensor, dest_loc: torch.Tensor, out: torch.Tensor, ctx: Optional[rt.Context] = None) -> torch.Tensor:

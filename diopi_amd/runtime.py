@@ -173,6 +173,8 @@ class _Libs:
         impl.diopiPromptFlashAttention.argtypes = [vp, vp, vp, vp, vp, vp, _SizeStruct, i64, i64, i64, i64]
         impl.diopiRootMeanSquareNormInp.argtypes = [vp, vp, vp, ctypes.c_float]
         impl.diopiFusedAddRootMeanSquareNormInp.argtypes = [vp, vp, vp, vp, vp, ctypes.c_float]
+        impl.diopiFusedDecoderAttentionInp.argtypes = [vp, vp, vp, vp, vp, ctypes.POINTER(i64), i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64,
+                                                       ctypes.c_float]
         for name in OPERATOR_SYMBOLS:
             getattr(impl, name).restype = i32
 
@@ -198,6 +200,7 @@ OPERATOR_SYMBOLS = (
     "diopiPromptFlashAttention",
     "diopiRootMeanSquareNormInp",
     "diopiFusedAddRootMeanSquareNormInp",
+    "diopiFusedDecoderAttentionInp",
 )
 INFO_SYMBOLS = ("diopiGetVendorName", "diopiGetImplVersion", "diopiGetLastErrorString")
 

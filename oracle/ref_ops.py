@@ -29,6 +29,8 @@ context_attention            functions_lightllm.cpp:109-147; customized_test.py:
 flash_attention              customized_test.py:462-485 (declaration functions_ext.h:209-212)
 flash_attention_varlen       customized_test.py:525-588 with multi_head_attention_inside, 36-57 (the torch
                              implementation calls the flash-attn library; declaration functions_ext.h:355-359)
+fused_decoder_attention_inp  proto/include/diopi/functions_lmdeploy.h:104-135 (prototype and five lines of prose; no
+                             implementation, Python statement or test case in the reference tree)
 prompt_flash_attention       customized_test.py:751-780 (no torch body; declaration functions_ext.h:684-686)
 paged_attention              customized_test.py:782-821 (no torch body; declaration functions_ext.h:616-618),
                              extended from its single in-order sequence to a block table per sequence
@@ -88,6 +90,15 @@ inside the 1e-2 bar of 16-bit tensors, and not at all in fp32 beyond 1e-6:
   paged_attention      the reference's case shape (diopi_configs.py:9425-9468: 5 tokens, blocks [0, 1]) against the
                        statement's own reading (rows 0..4), shuffled block tables against explicit Python loops in
                        float64, agreement with token_attention + token_softmax_reducev on the expanded row table
+  fused_decoder_attention_inp  a composition of parts pinned above: a matrix product in the tensor dtype, rotary_emb,
+                       token_attention and token_softmax_reducev on the window of the contiguous cache.  Pinned by:
+                       identity weights and zero position return the decode pair's result on the same rows; one cached
+                       token returns the projected v row; the cache rows written equal the projected k / v bit for bit;
+                       explicit Python loops in float64.  "Parity unpinned" (the header's prose does not decide them and
+                       the reference holds nothing else): the rotary pairing (half-split, as diopiRotaryEmbedding), the
+                       circular window once a sequence reaches max_seq_len, where the output lands when
+                       local_head_num * size_per_head < hidden_units, the treatment of finished rows, and where the 16-bit
+                       roundings fall (all inside the 1e-2 bar of 16-bit tensors)
   context_attention    first token of every sequence returns its v row bit for bit, constant V,
                        the reference's ragged fixtures (diopi_configs.py:9349-9377) incl. untouched
                        rows, float64 brute force, and the last row cross-checked against
@@ -468,3 +479,61 @@ def paged_attention(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
         V = v[rows].to(cdt).repeat_interleave(g, dim=1).view(1, L, numHeads, dim).transpose(1, 2)
         out[i] = torch.matmul(P, V).view(numHeads, dim)
     return out.to(query.dtype).view(-1, numHeads * dim)
+
+
+def fused_decoder_attention_inp(inoutput: torch.Tensor, qkv_weight: torch.Tensor, qkv_bias: Optional[torch.Tensor], key_cache: torch.Tensor,
+                                value_cache: torch.Tensor, finished: Optional[torch.Tensor], total_padding_tokens: Optional[torch.Tensor],
+                                sequence_lengths: torch.Tensor, step: int, layer_id: int, local_head_num: int, local_kv_head_num: int, size_per_head: int,
+                                max_seq_len: int, rotary_embedding: int, rope_theta: float, exact: bool = False) -> torch.Tensor:
+    """functions_lmdeploy.h:104-135, in place on key_cache / value_cache; returns the new inoutput (float64 when exact).
+
+    "1.get QKV": inoutput @ qkv_weight in the tensor dtype (+ qkv_bias).  "2.qkv add bias & apply rotary embedding, tstep =
+    step - 1 - padd_len": the half-split rotation of rotary_emb on every q and k head at that position, angles
+    pos * rope_theta^(-2j/rotary_embedding).  "4.Kv saved to cache ... cache index = seq%max_seq": row
+    sequence_lengths[b] % max_seq_len of [layer_id, b, kv head].  "3. ... softmax(QK)*V.qk *= inv_sqrt_dh ... eps = 1.e-6f":
+    token_attention and token_softmax_reducev over the last min(L + 1, max_seq_len) cached tokens, the eps added to the
+    softmax denominator.  Finished rows keep their inoutput and their cache rows."""
+    B, hidden = inoutput.shape
+    H, Hkv, D = local_head_num, local_kv_head_num, size_per_head
+    dt = inoutput.dtype
+    cdt = torch.float64 if exact else torch.float32
+    out = inoutput.to(torch.float64).clone() if exact else inoutput.clone()
+    if exact:
+        qkv = inoutput.double() @ qkv_weight.double()
+    else:
+        qkv = (inoutput.float() @ qkv_weight.float()).to(dt).float()  # the product as a matmul in the tensor dtype leaves it
+    if qkv_bias is not None:
+        qkv = qkv + qkv_bias.reshape(1, -1).to(cdt)
+    qkv = qkv.view(B, H + 2 * Hkv, D)
+    for b in range(B):
+        if finished is not None and bool(finished[b]):
+            continue
+        L = int(sequence_lengths[b])
+        pad = int(total_padding_tokens[b]) if total_padding_tokens is not None else 0
+        heads = qkv[b]
+        if rotary_embedding > 0:
+            j = torch.arange(rotary_embedding // 2, dtype=torch.float64)
+            ang = float(step - 1 - pad) * rope_theta ** (-2.0 * j / rotary_embedding)
+            cos, sin = ang.cos().to(cdt), ang.sin().to(cdt)
+            rot = rotary_emb(heads[: H + Hkv, :rotary_embedding], cos, sin, False, exact=exact).to(cdt)
+            heads = torch.cat((torch.cat((rot, heads[: H + Hkv, rotary_embedding:]), dim=-1), heads[H + Hkv:]), dim=0)
+        q = heads[:H] if exact else heads[:H].to(dt)
+        slot = L % max_seq_len
+        key_cache[layer_id, b, :, slot] = heads[H:H + Hkv].to(key_cache.dtype)
+        value_cache[layer_id, b, :, slot] = heads[H + Hkv:].to(value_cache.dtype)
+        n = min(L + 1, max_seq_len)
+        rows = ((torch.arange(L + 1 - n, L + 1)) % max_seq_len).to(torch.int32).reshape(1, n)
+        k_rows = key_cache[layer_id, b].transpose(0, 1).contiguous()    # [max_seq_len, Hkv, D]: a slot per cache row
+        v_rows = value_cache[layer_id, b].transpose(0, 1).contiguous()
+        logits = torch.zeros(H, n, dtype=torch.float64 if exact else dt)
+        token_attention(q.reshape(1, H, D), k_rows, logits, rows, torch.tensor([0]), torch.tensor([n]), n, exact=exact)
+        # softmax with the eps of the prose in the denominator: p = e / (sum e + 1e-6), e relative to the row maximum
+        lg = logits.to(cdt)
+        e = (lg - lg.max(-1, keepdim=True).values).exp()
+        p = e / (e.sum(-1, keepdim=True) + 1e-6)
+        if not exact:
+            p = p.to(dt)                                            # the probabilities meet V in the tensor dtype
+        V = v_rows[rows[0].long()].to(p.dtype).repeat_interleave(H // Hkv, dim=1).transpose(0, 1)  # [H, n, D]
+        o = torch.matmul(p.unsqueeze(1), V).reshape(H * D)
+        out[b, : H * D] = o.to(out.dtype)
+    return out

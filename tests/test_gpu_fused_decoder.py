@@ -1,0 +1,136 @@
+"""Parity of diopiFusedDecoderAttentionInp (called through the C ABI) against the CPU oracle's composition of the
+reference's pinned parts.  Bar: 16-bit tensors within atol = rtol = 1e-2 of the dtype-faithful composition and of float64;
+the cache rows the call writes are compared the same way, every other cache row bit for bit."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from diopi_amd import functions as F
+from diopi_amd import runtime as rt
+from oracle import ref_ops as O
+from tests.helpers import TOL, assert_bit_equal, assert_close, report
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _case(B, H, Hkv, S, seq, dt, seed, hidden=None, layers=2, layer=1, pad=None, finished=None, step=None, bias=True, rot=128, idt=torch.int32,
+          theta=10000.0, what=""):
+    D = 128
+    g = torch.Generator().manual_seed(seed)
+    hid = H * D if hidden is None else hidden
+    N = (H + 2 * Hkv) * D
+    x = torch.randn(B, hid, generator=g).to(dt)
+    w = (torch.randn(hid, N, generator=g) / math.sqrt(hid)).to(dt)
+    b = torch.randn(N, generator=g).to(dt) if bias else None
+    kc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dt)
+    vc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dt)
+    seq_t = torch.tensor(seq, dtype=idt)
+    pad_t = None if pad is None else torch.tensor(pad, dtype=idt)
+    fin_t = None if finished is None else torch.tensor(finished, dtype=torch.bool)
+    step = max(seq) + 1 if step is None else step
+    say("fused decoder attention", what, dict(B=B, H=H, Hkv=Hkv, S=S, hidden=hid, dtype=str(dt), seq=seq[:8], step=step))
+    # oracle, dtype-faithful and float64 (each on its own copy of the caches)
+    rk, rv = kc.clone(), vc.clone()
+    ref = O.fused_decoder_attention_inp(x, w, b, rk, rv, fin_t, pad_t, seq_t, step, layer, H, Hkv, D, S, rot, theta)
+    ek, ev = kc.double(), vc.double()
+    ex = O.fused_decoder_attention_inp(x, w, b, ek, ev, fin_t, pad_t, seq_t, step, layer, H, Hkv, D, S, rot, theta, exact=True)
+    # device
+    xd, wd, bd, kd, vd = x.to(DEV), w.to(DEV), (None if b is None else b.to(DEV)), kc.to(DEV), vc.to(DEV)
+    args = [t if t is None else t.to(DEV) for t in (fin_t, pad_t, seq_t)]
+    w_before = wd.clone()
+    out = F.fused_decoder_attention_inp(xd, wd, bd, None, 0, kd, vd, args[0], args[1], args[2], step, layer, H, Hkv, D, S, rot, theta)
+    assert_bit_equal(wd, w_before, "qkv_weight was modified")
+    tol = TOL[dt]
+    assert_close(out, ref, what=what + " output vs reference composition", **tol)
+    assert_close(out, ex, what=what + " output vs float64", **tol)
+    say(what, "max_abs/rel vs f64: %.3e %.3e" % report(out, ex))
+    # caches: the written rows within tolerance, every other row untouched
+    written = torch.zeros(layers, B, Hkv, S, dtype=torch.bool)
+    for i in range(B):
+        if finished is None or not finished[i]:
+            written[layer, i, :, seq[i] % S] = True
+    for name, dev, r, e, orig in (("key_cache", kd, rk, ek, kc), ("value_cache", vd, rv, ev, vc)):
+        devc = dev.cpu()
+        assert_bit_equal(devc[~written], orig[~written], f"{what}: {name} rows outside the insertion were modified")
+        assert_close(devc[written], r[written], what=f"{what} {name} new rows vs reference composition", **tol)
+        assert_close(devc[written], e[written], what=f"{what} {name} new rows vs float64", **tol)
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_decoder_attention_small(dtype):
+    # multi-head, one range; lengths 0 (nothing cached), mid, last row of the cache
+    _case(B=5, H=4, Hkv=4, S=64, seq=[0, 1, 31, 40, 63], dt=dtype, seed=1, what="MHA")
+    # grouped heads, several ranges (S > 256), int64 index tensors, padding offsets, a finished row, no bias
+    _case(B=4, H=8, Hkv=2, S=700, seq=[5, 300, 699, 450], dt=dtype, seed=2, pad=[0, 3, 10, 1], finished=[False, False, False, True], bias=False,
+          idt=torch.int64, what="GQA 4, ranges")
+    # multi-query, hidden wider than H*D, no rotation, layer 0
+    _case(B=3, H=16, Hkv=1, S=96, seq=[95, 10, 50], dt=dtype, seed=3, hidden=16 * 128 + 256, layer=0, rot=0, what="MQA 16, wide hidden")
+
+
+def test_fused_decoder_attention_circular_cache_and_many_rows():
+    # sequences past max_seq_len wrap around; more than 64 batch rows take a second row group of the projection
+    _case(B=70, H=4, Hkv=2, S=48, seq=[(7 * i) % 200 for i in range(70)], dt=torch.float16, seed=4, step=260, what="wrap, 70 rows")
+
+
+def test_fused_decoder_attention_decode_shape_sampled():
+    """The decode benchmark's shape (batch 64, 32 heads of 128, hidden 4096, lengths 512..2047 in a 2048-row cache): the whole
+    output against the oracle."""
+    g = torch.Generator().manual_seed(5)
+    seq = torch.randint(512, 2048, (64,), generator=g).tolist()
+    _case(B=64, H=32, Hkv=32, S=2048, seq=seq, dt=torch.float16, seed=5, layers=1, layer=0, what="decode shape")
+
+
+def test_fused_decoder_attention_workspace_protocol_and_errors():
+    impl = rt.libs().impl
+    ctx = rt.Context()
+    B, H, Hkv, D, S = 2, 4, 4, 128, 512
+    x = torch.randn(B, H * D, dtype=torch.float16, device=DEV)
+    w = torch.randn(H * D, 3 * H * D, dtype=torch.float16, device=DEV)
+    kc = torch.zeros(1, B, Hkv, S, D, dtype=torch.float16, device=DEV)
+    vc = torch.zeros_like(kc)
+    seq = torch.tensor([3, 9], dtype=torch.int32, device=DEV)
+    hx, hw, hk, hv, hs = (rt.Tensor(t) for t in (x, w, kc, vc, seq))
+    tail = (0, hk.handle, hv.handle, None, None, hs.handle, 10, 0, H, Hkv, D, S, D, 10000.0)
+    # size query: nothing is computed
+    size = ctypes.c_int64(-1)
+    x0 = x.clone()
+    assert impl.diopiFusedDecoderAttentionInp(ctx.handle, hx.handle, hw.handle, None, None, ctypes.byref(size), *tail) == 0
+    ctx.synchronize()
+    assert size.value >= B * H * D * 2 and torch.equal(x, x0) and int(kc.abs().sum()) == 0
+    # a workspace that is too small is refused with a message
+    small = torch.empty(16, dtype=torch.int8, device=DEV)
+    hsm = rt.Tensor(small)
+    sz = ctypes.c_int64(16)
+    assert impl.diopiFusedDecoderAttentionInp(ctx.handle, hx.handle, hw.handle, None, hsm.handle, ctypes.byref(sz), *tail) != 0
+    assert b"workspace" in impl.diopiGetLastErrorString()
+    # an exact-size workspace and the context's own scratch give the same bits
+    ws = torch.empty(size.value, dtype=torch.int8, device=DEV)
+    hws = rt.Tensor(ws)
+    x1, k1 = x.clone(), kc.clone()
+    hx1, hk1 = rt.Tensor(x1), rt.Tensor(k1)
+    assert impl.diopiFusedDecoderAttentionInp(ctx.handle, hx1.handle, hw.handle, None, hws.handle, ctypes.byref(size), *((0, hk1.handle) + tail[2:])) == 0
+    x2, k2 = x.clone(), kc.clone()
+    hx2, hk2 = rt.Tensor(x2), rt.Tensor(k2)
+    zero = ctypes.c_int64(0)
+    assert impl.diopiFusedDecoderAttentionInp(ctx.handle, hx2.handle, hw.handle, None, None, ctypes.byref(zero), *((0, hk2.handle) + tail[2:])) == 0
+    ctx.synchronize()
+    ctx.clear_tensors()
+    assert_bit_equal(x1, x2, "workspace tensor vs context scratch")
+    assert_bit_equal(k1, k2, "workspace tensor vs context scratch: key cache")
+    # shapes this build does not implement answer diopiNoImplement (13)
+    x64 = torch.randn(B, 4 * 64, dtype=torch.float16, device=DEV)
+    w64 = torch.randn(4 * 64, 3 * 4 * 64, dtype=torch.float16, device=DEV)
+    k64 = torch.zeros(1, B, 4, S, 64, dtype=torch.float16, device=DEV)
+    v64 = k64.clone()
+    hx64, hw64, hk64, hv64 = (rt.Tensor(t) for t in (x64, w64, k64, v64))
+    r = impl.diopiFusedDecoderAttentionInp(ctx.handle, hx64.handle, hw64.handle, None, None, ctypes.byref(ctypes.c_int64(-1)), 0, hk64.handle, hv64.handle,
+                                           None, None, hs.handle, 10, 0, 4, 4, 64, S, 64, 10000.0)
+    assert r == 13, r

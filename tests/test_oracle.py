@@ -704,3 +704,102 @@ def test_paged_attention_reference_case_and_block_tables():
     out = torch.zeros(B, H, D, dtype=torch.float64)
     O.token_softmax_reducev(logits, v.view(-1, Hkv, D), out, b_loc, start, blen, maxlen, 0, exact=True)
     assert_close(got.view(B, H, D), out, 1e-12, 1e-12, "paged attention vs token_attention + token_softmax_reducev")
+
+
+# ----------------------------------------------------------------------------- fused decoder attention (lmdeploy set)
+def _fused_inputs(seed, B, H, Hkv, D, S, layers=2, dtype=torch.float64, bias=True):
+    g = rng(seed)
+    hid, N = H * D, (H + 2 * Hkv) * D
+    x = torch.randn(B, hid, generator=g).to(dtype)
+    w = (torch.randn(hid, N, generator=g) / math.sqrt(hid)).to(dtype)
+    b = torch.randn(N, generator=g).to(dtype) if bias else None
+    kc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dtype)
+    vc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dtype)
+    return x, w, b, kc, vc
+
+
+def test_fused_decoder_attention_python_loops():
+    """Every step of the header's prose written out with explicit loops in float64 (functions_lmdeploy.h:104-135)."""
+    B, H, Hkv, D, S = 3, 4, 2, 8, 6
+    x, w, b, kc, vc = _fused_inputs(40, B, H, Hkv, D, S)
+    seq = torch.tensor([0, 3, 9])          # the last one has wrapped around the 6-row cache
+    pad = torch.tensor([0, 1, 2])
+    fin = torch.tensor([False, False, False])
+    step, layer, theta = 12, 1, 10000.0
+    kc2, vc2 = kc.clone(), vc.clone()
+    got = O.fused_decoder_attention_inp(x, w, b, kc2, vc2, fin, pad, seq, step, layer, H, Hkv, D, S, D, theta, exact=True)
+    G = H // Hkv
+    for bi in range(B):
+        qkv = [sum(float(x[bi, i]) * float(w[i, n]) for i in range(H * D)) + float(b[n]) for n in range((H + 2 * Hkv) * D)]
+        pos = step - 1 - int(pad[bi])
+        heads = [qkv[h * D:(h + 1) * D] for h in range(H + 2 * Hkv)]
+        for h in range(H + Hkv):           # q and k heads rotate, v heads do not
+            r = list(heads[h])
+            for j in range(D // 2):
+                ang = pos * theta ** (-2.0 * j / D)
+                r[j] = heads[h][j] * math.cos(ang) - heads[h][j + D // 2] * math.sin(ang)
+                r[j + D // 2] = heads[h][j] * math.sin(ang) + heads[h][j + D // 2] * math.cos(ang)
+            heads[h] = r
+        L = int(seq[bi])
+        slot = L % S
+        for hk in range(Hkv):
+            assert_close(kc2[layer, bi, hk, slot], torch.tensor(heads[H + hk], dtype=torch.float64), 1e-12, 1e-12, "cached k row")
+            assert_close(vc2[layer, bi, hk, slot], torch.tensor(heads[H + Hkv + hk], dtype=torch.float64), 1e-12, 1e-12, "cached v row")
+        toks = [t % S for t in range(max(0, L + 1 - S), L + 1)]
+        for h in range(H):
+            hk = h // G
+            sc = [sum(heads[h][d] * float(kc2[layer, bi, hk, t, d]) for d in range(D)) / math.sqrt(D) for t in toks]
+            m = max(sc)
+            e = [math.exp(s_ - m) for s_ in sc]
+            den = sum(e) + 1e-6
+            for d in range(D):
+                want = sum(e[i] / den * float(vc2[layer, bi, hk, t, d]) for i, t in enumerate(toks))
+                assert abs(float(got[bi, h * D + d]) - want) < 1e-10, (bi, h, d)
+    # every other cache row and the other layer are untouched
+    keep = torch.ones_like(kc, dtype=torch.bool)
+    for bi in range(B):
+        keep[layer, bi, :, int(seq[bi]) % S] = False
+    assert torch.equal(kc2[keep], kc[keep]) and torch.equal(vc2[keep], vc[keep])
+
+
+def test_fused_decoder_attention_reduces_to_the_decode_pair():
+    """An identity projection at rotary position 0 leaves q, k, v equal to slices of the input: the result must then be
+    token_attention + token_softmax_reducev (both pinned above) on the cache rows, for the dtype-faithful mode too."""
+    B, H, D, S = 2, 2, 8, 16
+    Hkv = H
+    for dt in (torch.float64, torch.float16):
+        g = rng(41)
+        hid = 3 * H * D
+        x = torch.randn(B, hid, generator=g).to(dt)
+        w = torch.eye(hid).to(dt)          # q = x[:, :HD], k = x[:, HD:2HD], v = x[:, 2HD:]
+        kc = torch.randn(1, B, Hkv, S, D, generator=g).to(dt)
+        vc = torch.randn(1, B, Hkv, S, D, generator=g).to(dt)
+        seq = torch.tensor([4, 7])
+        kc2, vc2 = kc.clone(), vc.clone()
+        got = O.fused_decoder_attention_inp(x, w, None, kc2, vc2, None, None, seq, 1, 0, H, Hkv, D, S, D, 10000.0, exact=dt == torch.float64)
+        for bi in range(B):
+            n = int(seq[bi]) + 1
+            assert_bit_equal(kc2[0, bi, :, n - 1], x[bi, H * D:2 * H * D].view(Hkv, D), "position 0 and identity weights: k row is the input slice")
+            loc = torch.arange(n, dtype=torch.int32).reshape(1, n)
+            krows, vrows = kc2[0, bi].transpose(0, 1).contiguous(), vc2[0, bi].transpose(0, 1).contiguous()
+            lg = torch.zeros(H, n, dtype=dt)
+            O.token_attention(x[bi, :H * D].view(1, H, D), krows, lg, loc, torch.tensor([0]), torch.tensor([n]), n, exact=dt == torch.float64)
+            o = torch.zeros(1, H, D, dtype=dt)
+            O.token_softmax_reducev(lg, vrows, o, loc, torch.tensor([0]), torch.tensor([n]), n, 0, exact=dt == torch.float64)
+            # the eps of the fused form moves the probabilities by at most 1e-6 relative
+            tol = dict(rtol=2e-6, atol=1e-9) if dt == torch.float64 else dict(rtol=1e-2, atol=1e-2)
+            assert_close(got[bi, :H * D].view(H, D), o[0], what=f"fused vs decode pair {dt}", **tol)
+            assert_bit_equal(got[bi, H * D:].to(dt), x[bi, H * D:], "columns past H*D keep their values")
+
+
+def test_fused_decoder_attention_first_token_and_finished_rows():
+    """With nothing cached the output is the projected v row itself (softmax over one token, up to the eps); a finished row
+    keeps its hidden state and its cache rows."""
+    B, H, Hkv, D, S = 2, 4, 1, 8, 4
+    x, w, b, kc, vc = _fused_inputs(42, B, H, Hkv, D, S, layers=1)
+    kc2, vc2 = kc.clone(), vc.clone()
+    got = O.fused_decoder_attention_inp(x, w, b, kc2, vc2, torch.tensor([False, True]), None, torch.tensor([0, 2]), 1, 0, H, Hkv, D, S, D, 10000.0, exact=True)
+    v_row = (x[0] @ w + b)[(H + Hkv) * D:]
+    for h in range(H):
+        assert_close(got[0, h * D:(h + 1) * D], v_row / (1 + 1e-6), 1e-12, 1e-12, "one token: its v row")
+    assert torch.equal(got[1], x[1]) and torch.equal(kc2[0, 1], kc[0, 1]) and torch.equal(vc2[0, 1], vc[0, 1])
