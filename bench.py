@@ -415,7 +415,46 @@ def main():
         e_pg = record("diopiPagedAttention (blocks of 128 rows)", f"cfg3 lengths fp16 B={B3}", ms_pg, head["b_att"] + head["b_red"], "hbm", "f16", None,
                       note="widening beyond the seven hot-path operators; block table -> row table, then the two decode kernels")
         e_pg["tokens_per_s"] = round(B3 / (ms_pg * 1e-3), 1)
-        del w3, src, perm, hsrc, hperm, hcache, hp, q2, k2, v2, o2, table
+        del src, perm, hsrc, hperm, hcache, hp, q2, k2, v2, o2, table
+        torch.cuda.empty_cache()
+        # the same decode step behind the fused lmdeploy interface: QKV projection of [64, 4096] hidden states, bias, rotary,
+        # cache insertion and attention over contiguous per-sequence caches [1, 64, 32, 2048, 128] with the cfg3 lengths
+        # (one token fewer cached, so that the window of every row is its cfg3 length); no logits tensor exists
+        hid, S3 = H3 * D3, 2048
+        N3 = 3 * H3 * D3
+        g3 = torch.Generator(device=dev)
+        g3.manual_seed(33)
+        xs = [(torch.randn(B3, hid, device=dev, generator=g3) * 0.5).to(torch.float16) for _ in range(3)]
+        wq = (torch.randn(hid, N3, device=dev, generator=g3) / math.sqrt(hid)).to(torch.float16)
+        bq = torch.randn(N3, device=dev, generator=g3).to(torch.float16)
+        kcs = w3["k_cache"].view(1, B3, S3, H3, D3).permute(0, 1, 3, 2, 4).contiguous()
+        vcs = w3["v_cache"].view(1, B3, S3, H3, D3).permute(0, 1, 3, 2, 4).contiguous()
+        cached = (w3["b_seq_len"] - 1).to(torch.int32)
+        hfz = {k: Tensor(v) for k, v in dict(w=wq, b=bq, k=kcs, v=vcs, s=cached).items()}
+        hxs = [Tensor(x) for x in xs]
+        size = ctypes.c_int64(-1)
+        check(impl.diopiFusedDecoderAttentionInp(ctx.handle, hxs[0].handle, hfz["w"].handle, hfz["b"].handle, None, ctypes.byref(size), 0, hfz["k"].handle,
+                                                 hfz["v"].handle, None, None, hfz["s"].handle, 2048, 0, H3, H3, D3, S3, D3, 10000.0), "size query")
+        wsp = torch.empty(int(size.value), dtype=torch.int8, device=dev)
+        hwsp = Tensor(wsp)
+
+        def fused(i):
+            check(impl.diopiFusedDecoderAttentionInp(ctx.handle, hxs[i % 3].handle, hfz["w"].handle, hfz["b"].handle, hwsp.handle, ctypes.byref(size), 0,
+                                                     hfz["k"].handle, hfz["v"].handle, None, None, hfz["s"].handle, 2048, 0, H3, H3, D3, S3, D3, 10000.0),
+                  "diopiFusedDecoderAttentionInp")
+
+        ms_fz = timed(fused)
+        kv_rows = int(w3["b_seq_len"].sum())
+        b_proj = hid * N3 * 2 + N3 * 2 + B3 * hid * 2 + B3 * N3 * 2            # weights, bias, hidden states in, q / new k / new v out
+        b_attn = kv_rows * 2 * H3 * D3 * 2 + B3 * H3 * D3 * 2 * 2 + 4 * B3    # one K and one V row per cached token, q in, output, lengths
+        e_fz = record("diopiFusedDecoderAttentionInp (projection + rotary + cache insert + attention)", f"cfg3 lengths fp16 B={B3} hidden={hid}", ms_fz,
+                      b_proj + b_attn, "hbm", "f16", None,
+                      note="widening (lmdeploy set): the decode step without a logits tensor; bytes = projection weights once + one K and one V row "
+                           "per cached token; compare its attention share with TokenAttention + TokenSoftmaxReduceV above, which move the same rows "
+                           "plus the logits twice")
+        e_fz["tokens_per_s"] = round(B3 / (ms_fz * 1e-3), 1)
+        e_fz["projection_bytes"], e_fz["attention_bytes"] = int(b_proj), int(b_attn)
+        del w3, xs, wq, bq, kcs, vcs, hfz, hxs, wsp, hwsp
         torch.cuda.empty_cache()
 
     if not only or "cfg5" in only:

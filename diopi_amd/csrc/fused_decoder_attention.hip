@@ -16,14 +16,17 @@
 // Open in the prose, fixed here: the rotary pairing (2), a circular cache window once L reaches max_seq_len (3, 4),
 // where the output lands when H*D < hidden_units (5), and that finished rows are left untouched everywhere.
 //
-// Three kernels, all on the context's stream:
+// Three kernels (four when the projection's hidden dimension is split), all on the context's stream:
 //   fusedQkvHead     one work-group per head of the projection (128 output columns) and 64 batch rows.  The weight
-//                    panel [hidden, 128] is streamed once: 8 waves = 4 row blocks of 16 batch rows x 2 halves of the
-//                    hidden dimension.  A lane loads 8 consecutive weight rows (16 bytes = 8 columns each); pairs of rows
+//                    panel [hidden, 128] goes through 8 waves = 4 quarters of the hidden dimension x 2 halves of the batch
+//                    rows.  A lane loads 8 consecutive weight rows (16 bytes = 8 columns each); pairs of rows
 //                    interleaved with two byte permutes become the B operands of v_mfma_f32_16x16x32 for the lane's 8
-//                    columns, the A operand is 16 bytes of a hidden-state row.  The two halves meet in LDS (fp32), and
+//                    columns and serve two products (two blocks of 16 batch rows, whose A operands are 16 bytes of a
+//                    hidden-state row each).  The quarters meet in LDS (fp32), and
 //                    the same work-group adds the bias, rotates, and writes the head: q to the workspace, k and v
-//                    straight into the cache.  HBM-bound on the weights.
+//                    straight into the cache.  HBM-bound on the weights.  With few heads and rows the hidden dimension is
+//                    also cut across work-groups (up to one work-group per compute unit in all); their fp32 sums then go
+//                    through the workspace and fusedQkvFinish adds them and does the bias, rotation and stores.
 //   fusedDecodeAttn  a wave owns (batch row, kv head, range of cached tokens): per 32 tokens 8 K loads that arrive in
 //                    the B-operand layout of q.k^T (16 lanes x 16-byte pieces of 16 consecutive cache rows), online
 //                    softmax on the 16 x 32 scores (row maxima and sums by DPP row reductions), probabilities through a
@@ -42,7 +45,8 @@ namespace {
 
 constexpr int kFD = 128;          // head size of the fast path
 constexpr int kProjThreads = 512;
-constexpr int kProjSlabs = kProjThreads / kWave / 4;  // slabs of the hidden dimension: waves = 4 row blocks x slabs
+constexpr int kProjRB = 2;         // blocks of 16 batch rows per wave
+constexpr int kProjSlabs = kProjThreads / kWave / 2;  // slabs of the hidden dimension: waves = 2 row halves x slabs
 constexpr int kProjRows = 64;     // batch rows per work-group of the projection
 constexpr int kProjPitch = kFD + 4;  // floats per row of a partial tile: rows 4 apart are 16 banks apart
 constexpr int kAttnThreads = 256;
@@ -71,50 +75,89 @@ __device__ __forceinline__ int64_t rowLength(const FusedArgs& a, int b) {
     return L < 0 ? 0 : L;
 }
 
+// Finishes the pair (j, j + 64) of head `tile` of batch row b from the fp32 sums of the projection: rounding of the product,
+// bias, rotation, and the store to where the head belongs (q to the workspace, k and v into the cache row of the new token).
+template <typename T>
+__device__ __forceinline__ void finishPair(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const T* __restrict__ bias, const FusedArgs& a,
+                                           int tile, int b, int j, float v0, float v1) {
+    const bool isQ = tile < a.H;
+    const bool isK = !isQ && tile < a.H + a.Hkv;
+    const int head = isQ ? tile : (isK ? tile - a.H : tile - a.H - a.Hkv);
+    // the product is rounded to the element type as a matrix product in that type would leave it
+    float y0 = toFloat(fromFloat<T>(v0)), y1 = toFloat(fromFloat<T>(v1));
+    if (bias != nullptr) {
+        y0 += toFloat(bias[tile * kFD + j]);
+        y1 += toFloat(bias[tile * kFD + j + kFD / 2]);
+    }
+    if ((isQ || isK) && a.rot > 0) {
+        const int64_t pad = a.padding != nullptr ? loadIndex(a.padding, b, a.pad64) : 0;
+        const float pos = static_cast<float>(a.step - 1 - pad);
+        const float invFreq = exp2f(-(2.0f * static_cast<float>(j) / static_cast<float>(a.rot)) * log2f(a.ropeTheta));
+        float sn, cs;
+        sincosf(pos * invFreq, &sn, &cs);
+        const float o0 = y0 * cs - y1 * sn;
+        const float o1 = y0 * sn + y1 * cs;
+        y0 = o0;
+        y1 = o1;
+    }
+    T* dst;
+    if (isQ) {
+        dst = qOut + (static_cast<int64_t>(b) * a.H + head) * kFD;
+    } else {
+        const int64_t slot = rowLength(a, b) % a.maxSeq;
+        dst = (isK ? kCache : vCache) + a.layerOffset + ((static_cast<int64_t>(b) * a.Hkv + head) * a.maxSeq + slot) * kFD;
+    }
+    dst[j] = fromFloat<T>(y0);
+    dst[j + kFD / 2] = fromFloat<T>(y1);
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const T* __restrict__ x,
-                                                            const T* __restrict__ w, const T* __restrict__ bias, FusedArgs a) {
+__global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, float* __restrict__ hiddenPart,
+                                                            const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, FusedArgs a) {
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
-    extern __shared__ __attribute__((aligned(16))) float part[];  // [kProjSlabs][64 rows][kProjPitch]
+    extern __shared__ __attribute__((aligned(16))) float part[];  // [kProjSlabs / 2][64 rows][kProjPitch]
     const int tile = blockIdx.x;  // head of the projection: H query heads, then Hkv key heads, then Hkv value heads
     const int rowBase = blockIdx.y * kProjRows;
     const int N = (a.H + 2 * a.Hkv) * kFD;
     const int lane = threadIdx.x % kWave;
-    const int wave = threadIdx.x / kWave;
-    const int rb = wave % 4;   // block of 16 batch rows
-    const int ks = wave / 4;   // slab of the hidden dimension
+    const int rh = (threadIdx.x / kWave) % 2;  // half of the 64 batch rows
+    const int ks = threadIdx.x / kWave / 2;    // slab of the hidden dimension
     const int g4 = lane / 16;  // A, B: k slots 8 g4 .. + 7 of a 32-row step; C: rows 4 g4 .. + 3
-    const int c = lane % 16;   // A: batch row of the block; loads: 16-byte packet (8 columns) of the panel; C: column
-    const int kPer = a.hidden / kProjSlabs;  // a multiple of 32
+    const int c = lane % 16;   // A: batch row of a block; loads: 16-byte packet (8 columns) of the panel; C: column
+    const int kPer = a.hidden / (kProjSlabs * gridDim.z);  // a multiple of 32
     const int steps = kPer / 32;
-    int row = rowBase + rb * 16 + c;
-    row = row < a.B ? row : a.B - 1;
-    const T* xRow = x + static_cast<int64_t>(row) * a.hidden + ks * kPer + 8 * g4;
-    const T* wCol = w + static_cast<int64_t>(ks * kPer + 8 * g4) * N + tile * kFD + 8 * c;
-
-    f32x4 acc[8];
+    const int kBeg = (blockIdx.z * kProjSlabs + ks) * kPer;
+    const T* xRow[kProjRB];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < kProjRB; ++rb) {
+        int row = rowBase + (rh * kProjRB + rb) * 16 + c;
+        row = row < a.B ? row : a.B - 1;
+        xRow[rb] = x + static_cast<int64_t>(row) * a.hidden + kBeg + 8 * g4;
+    }
+    const T* wCol = w + static_cast<int64_t>(kBeg + 8 * g4) * N + tile * kFD + 8 * c;
+
+    f32x4 acc[kProjRB][8];
+#pragma unroll
+    for (int rb = 0; rb < kProjRB; ++rb) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[rb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     struct Step {
         u32x4 w[8];
-        u32x4 x;
+        u32x4 x[kProjRB];
     };
     // every step issues the same loads (past the last step the last one again), so that the wait for one step's rows
     // leaves exactly the next step's in flight
     auto issue = [&](int s, Step& st) {
         const int sc = s < steps ? s : steps - 1;
-        st.x = *reinterpret_cast<const u32x4*>(xRow + 32 * sc);
 #pragma unroll
         for (int r = 0; r < 8; ++r) st.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wCol + static_cast<int64_t>(32 * sc + r) * N));
+#pragma unroll
+        for (int rb = 0; rb < kProjRB; ++rb) st.x[rb] = *reinterpret_cast<const u32x4*>(xRow[rb] + 32 * sc);
     };
     auto consume = [&](const Step& st) {
-        union {
-            u32x4 u;
-            Frag f;
-        } pa;
-        pa.u = st.x;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             union {
@@ -127,8 +170,16 @@ __global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOu
                 lo.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x05040100u);
                 hi.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x07060302u);
             }
-            acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
-            acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
+#pragma unroll
+            for (int rb = 0; rb < kProjRB; ++rb) {
+                union {
+                    u32x4 u;
+                    Frag f;
+                } pa;
+                pa.u = st.x[rb];
+                acc[rb][2 * j] = Ops::mma(pa.f, lo.f, acc[rb][2 * j]);
+                acc[rb][2 * j + 1] = Ops::mma(pa.f, hi.f, acc[rb][2 * j + 1]);
+            }
         }
     };
     Step sa, sb;
@@ -140,19 +191,50 @@ __global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOu
         if (s + 1 < steps) consume(sb);
         issue(s + 3, sb);
     }
-    // acc[e][r] is the sum of this slab for batch row rb*16 + 4 g4 + r, column 8c + e
-    float* mine = part + (ks * kProjRows + rb * 16 + 4 * g4) * kProjPitch + 8 * c;
+    // acc[rb][e][r] is the sum of this slab for batch row (rh*2 + rb)*16 + 4 g4 + r, column 8c + e.  The slabs meet in LDS in two
+    // rounds: the upper half of the waves writes, the lower half adds its own values to the same places.
+    float* mine = part + ((ks % (kProjSlabs / 2)) * kProjRows + rh * kProjRB * 16 + 4 * g4) * kProjPitch + 8 * c;
+    if (ks >= kProjSlabs / 2) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        *reinterpret_cast<f32x4*>(mine + r * kProjPitch) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-        *reinterpret_cast<f32x4*>(mine + r * kProjPitch + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+        for (int rb = 0; rb < kProjRB; ++rb) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* p = mine + (rb * 16 + r) * kProjPitch;
+                *reinterpret_cast<f32x4*>(p) = f32x4{acc[rb][0][r], acc[rb][1][r], acc[rb][2][r], acc[rb][3][r]};
+                *reinterpret_cast<f32x4*>(p + 4) = f32x4{acc[rb][4][r], acc[rb][5][r], acc[rb][6][r], acc[rb][7][r]};
+            }
+        }
+    }
+    __syncthreads();
+    if (ks < kProjSlabs / 2) {
+#pragma unroll
+        for (int rb = 0; rb < kProjRB; ++rb) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float* p = mine + (rb * 16 + r) * kProjPitch;
+                const f32x4 u0 = *reinterpret_cast<const f32x4*>(p), u1 = *reinterpret_cast<const f32x4*>(p + 4);
+                *reinterpret_cast<f32x4*>(p) = f32x4{acc[rb][0][r], acc[rb][1][r], acc[rb][2][r], acc[rb][3][r]} + u0;
+                *reinterpret_cast<f32x4*>(p + 4) = f32x4{acc[rb][4][r], acc[rb][5][r], acc[rb][6][r], acc[rb][7][r]} + u1;
+            }
+        }
     }
     __syncthreads();
 
+    if (gridDim.z > 1) {
+        // this work-group only saw a part of the hidden dimension: its sums go to the workspace, the finishing kernel adds
+        // the parts
+        float* dst = hiddenPart + (static_cast<int64_t>(blockIdx.z) * a.B) * N + tile * kFD;
+        for (int idx = threadIdx.x; idx < kProjRows * kFD; idx += kProjThreads) {
+            const int r = idx / kFD, col = idx % kFD;
+            if (rowBase + r >= a.B) continue;
+            float v = 0.f;
+#pragma unroll
+            for (int k4 = 0; k4 < kProjSlabs / 2; ++k4) v += part[(k4 * kProjRows + r) * kProjPitch + col];
+            dst[static_cast<int64_t>(rowBase + r) * N + col] = v;
+        }
+        return;
+    }
     // ---- bias, rotation, and the head's destination: a thread takes the pair (j, j + 64) of a batch row
-    const bool isQ = tile < a.H;
-    const bool isK = !isQ && tile < a.H + a.Hkv;
-    const int head = isQ ? tile : (isK ? tile - a.H : tile - a.H - a.Hkv);
     for (int idx = threadIdx.x; idx < kProjRows * (kFD / 2); idx += kProjThreads) {
         const int r = idx / (kFD / 2);
         const int j = idx % (kFD / 2);
@@ -160,36 +242,32 @@ __global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOu
         if (b >= a.B || rowFinished(a, b)) continue;
         float v0 = 0.f, v1 = 0.f;
 #pragma unroll
-        for (int k4 = 0; k4 < kProjSlabs; ++k4) {
+        for (int k4 = 0; k4 < kProjSlabs / 2; ++k4) {
             v0 += part[(k4 * kProjRows + r) * kProjPitch + j];
             v1 += part[(k4 * kProjRows + r) * kProjPitch + j + kFD / 2];
         }
-        // the product is rounded to the element type as a matrix product in that type would leave it
-        float y0 = toFloat(fromFloat<T>(v0)), y1 = toFloat(fromFloat<T>(v1));
-        if (bias != nullptr) {
-            y0 += toFloat(bias[tile * kFD + j]);
-            y1 += toFloat(bias[tile * kFD + j + kFD / 2]);
+        finishPair<T>(qOut, kCache, vCache, bias, a, tile, b, j, v0, v1);
+    }
+}
+
+// The second half of a projection whose hidden dimension was split over several work-groups per head: adds the parts and
+// finishes every pair as fusedQkvHead does.
+template <typename T>
+__global__ __launch_bounds__(256) void fusedQkvFinish(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const float* __restrict__ hiddenPart,
+                                                      const T* __restrict__ bias, FusedArgs a, int parts) {
+    const int tile = blockIdx.x;
+    const int N = (a.H + 2 * a.Hkv) * kFD;
+    for (int idx = threadIdx.x; idx < 4 * (kFD / 2); idx += 256) {
+        const int b = blockIdx.y * 4 + idx / (kFD / 2);
+        const int j = idx % (kFD / 2);
+        if (b >= a.B || rowFinished(a, b)) continue;
+        float v0 = 0.f, v1 = 0.f;
+        for (int p = 0; p < parts; ++p) {
+            const float* src = hiddenPart + (static_cast<int64_t>(p) * a.B + b) * N + tile * kFD;
+            v0 += src[j];
+            v1 += src[j + kFD / 2];
         }
-        if ((isQ || isK) && a.rot > 0) {
-            const int64_t pad = a.padding != nullptr ? loadIndex(a.padding, b, a.pad64) : 0;
-            const float pos = static_cast<float>(a.step - 1 - pad);
-            const float invFreq = exp2f(-(2.0f * static_cast<float>(j) / static_cast<float>(a.rot)) * log2f(a.ropeTheta));
-            float sn, cs;
-            sincosf(pos * invFreq, &sn, &cs);
-            const float o0 = y0 * cs - y1 * sn;
-            const float o1 = y0 * sn + y1 * cs;
-            y0 = o0;
-            y1 = o1;
-        }
-        T* dst;
-        if (isQ) {
-            dst = qOut + (static_cast<int64_t>(b) * a.H + head) * kFD;
-        } else {
-            const int64_t slot = rowLength(a, b) % a.maxSeq;
-            dst = (isK ? kCache : vCache) + a.layerOffset + ((static_cast<int64_t>(b) * a.Hkv + head) * a.maxSeq + slot) * kFD;
-        }
-        dst[j] = fromFloat<T>(y0);
-        dst[j + kFD / 2] = fromFloat<T>(y1);
+        finishPair<T>(qOut, kCache, vCache, bias, a, tile, b, j, v0, v1);
     }
 }
 
@@ -392,17 +470,26 @@ __global__ __launch_bounds__(256) void fusedDecodeMerge(T* __restrict__ out, Fus
 
 template <typename T>
 diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const void* bias, void* workspace, void* kCache, void* vCache, const FusedArgs& a,
-                         const AttnSplit& spIn, int64_t qBytes) {
+                         const AttnSplit& spIn, int64_t qBytes, int projParts) {
     T* qBuf = static_cast<T*>(workspace);
     AttnSplit sp = spIn;
-    sp.partAcc = reinterpret_cast<float*>(static_cast<char*>(workspace) + qBytes);
+    // the parts of a split projection share the storage of the attention partials: the attention kernel runs after the
+    // finishing kernel has read them
+    float* hiddenPart = reinterpret_cast<float*>(static_cast<char*>(workspace) + qBytes);
+    sp.partAcc = hiddenPart;
     sp.partMl = sp.partAcc + static_cast<int64_t>(a.B) * sp.splits * a.H * kFD;
-    const size_t projLds = static_cast<size_t>(kProjSlabs) * kProjRows * kProjPitch * sizeof(float);
+    const size_t projLds = static_cast<size_t>(kProjSlabs / 2) * kProjRows * kProjPitch * sizeof(float);
     ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(fusedQkvHead<T>), static_cast<int>(projLds)));
-    const dim3 pgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, kProjRows)));
-    hipLaunchKernelGGL((fusedQkvHead<T>), pgrid, dim3(kProjThreads), projLds, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache),
+    const dim3 pgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, kProjRows)), static_cast<unsigned>(projParts));
+    hipLaunchKernelGGL((fusedQkvHead<T>), pgrid, dim3(kProjThreads), projLds, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache), hiddenPart,
                        static_cast<const T*>(inout), static_cast<const T*>(w), static_cast<const T*>(bias), a);
     ROCM_LAUNCH_CHECK();
+    if (projParts > 1) {
+        const dim3 fgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, 4)));
+        hipLaunchKernelGGL((fusedQkvFinish<T>), fgrid, dim3(256), 0, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache), hiddenPart,
+                           static_cast<const T*>(bias), a, projParts);
+        ROCM_LAUNCH_CHECK();
+    }
     const dim3 agrid(static_cast<unsigned>(ceilDiv(a.Hkv, kAttnWaves)), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
     hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), 0, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
                        static_cast<const T*>(vCache), a, sp);
@@ -476,7 +563,7 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
         a.pad64 = vP.dtype == diopi_dtype_int64;
     }
     // what this build implements: 16-bit elements, heads of 128, up to 16 query heads per kv head, rotation of the whole head
-    // or none, a hidden size the projection's slabs of 32-row steps divide, 16-byte aligned rows
+    // or none, a hidden size that the projection's 4 slabs of 32-row steps divide, 16-byte aligned rows
     const bool supported = (vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16) && D == kFD && H / Hkv <= 16 &&
                            (rotary_embedding == 0 || rotary_embedding == kFD) && hidden % 128 == 0 && hidden >= 256 &&
                            ((reinterpret_cast<uintptr_t>(vX.data) | reinterpret_cast<uintptr_t>(vW.data) | reinterpret_cast<uintptr_t>(vK.data) |
@@ -499,8 +586,18 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
                static_cast<long long>(max_seq_len));
     const int64_t e = vX.itemsize();
     const int64_t qBytes = ceilDiv(B * H * D * e, 256) * 256;
-    const int64_t partBytes = sp.splits > 1 ? B * sp.splits * H * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
-    const int64_t need = qBytes + partBytes;
+    const int64_t attnBytes = sp.splits > 1 ? B * sp.splits * H * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
+    // work-groups of the projection per head: the hidden dimension is cut in two as long as that does not give more
+    // work-groups than compute units (measured at 96 heads x 64 rows x 4096: 2 parts 26 us faster than 1, 4 and 8 no better;
+    // a part must still give each of a work-group's 4 slabs whole 32-row steps)
+    int projParts = 1;
+    while (projParts < 8 && (H + 2 * Hkv) * ceilDiv(B, kProjRows) * projParts * 2 <= deviceInfo().numCU && hidden % (projParts * 2 * kProjSlabs * 32) == 0 &&
+           hidden / (projParts * 2 * kProjSlabs * 32) >= 2)
+        projParts *= 2;
+    projParts = envInt("DIOPI_ROCM_FUSEDDEC_PARTS", projParts);
+    if (projParts < 1 || hidden % (projParts * kProjSlabs * 32) != 0) projParts = 1;
+    const int64_t projBytes = projParts > 1 ? projParts * B * N * static_cast<int64_t>(sizeof(float)) : 0;
+    const int64_t need = qBytes + (attnBytes > projBytes ? attnBytes : projBytes);
     if (*workspace_size < 0) {
         *workspace_size = need;  // size query: nothing else happens
         return diopiSuccess;
@@ -531,8 +628,8 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     a.layerOffset = layer_id * B * Hkv * max_seq_len * D;
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes);
-    return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes);
+    if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, projParts);
+    return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, projParts);
 }
 
 }  // namespace

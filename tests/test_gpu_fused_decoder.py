@@ -71,6 +71,8 @@ def test_fused_decoder_attention_small(dtype):
     # grouped heads, several ranges (S > 256), int64 index tensors, padding offsets, a finished row, no bias
     _case(B=4, H=8, Hkv=2, S=700, seq=[5, 300, 699, 450], dt=dtype, seed=2, pad=[0, 3, 10, 1], finished=[False, False, False, True], bias=False,
           idt=torch.int64, what="GQA 4, ranges")
+    # three query heads on one kv head; a hidden size the projection cannot cut across work-groups (384 = 3 x 128)
+    _case(B=6, H=3, Hkv=1, S=40, seq=[0, 39, 7, 20, 33, 12], dt=dtype, seed=6, what="GQA 3, hidden 384")
     # multi-query, hidden wider than H*D, no rotation, layer 0
     _case(B=3, H=16, Hkv=1, S=96, seq=[95, 10, 50], dt=dtype, seed=3, hidden=16 * 128 + 256, layer=0, rot=0, what="MQA 16, wide hidden")
 
