@@ -40,16 +40,24 @@ class _on_stream:
 
     def __init__(self, ctx: rt.Context, *tensors):
         self.ctx = ctx
-        self.cuda = ctx.torch_stream is not None and any(t is not None and t.is_cuda for t in tensors)
+        on_device = any(t is not None and t.is_cuda for t in tensors)
+        self.cuda = ctx.torch_stream is not None and on_device
+        # a context that made its own native stream has no torch stream to order against: the host waits instead, before
+        # the call for what torch has queued (fills and copies of the arguments) and after it for the operator
+        self.foreign = ctx.torch_stream is None and on_device
 
     def __enter__(self):
         if self.cuda:
             self.ctx.torch_stream.wait_stream(torch.cuda.current_stream())
+        elif self.foreign:
+            torch.cuda.current_stream().synchronize()
         return self
 
     def __exit__(self, *exc):
         if self.cuda:
             torch.cuda.current_stream().wait_stream(self.ctx.torch_stream)
+        elif self.foreign:
+            self.ctx.synchronize()
         # scratch an operator took from the context (partial sums, tile plans, score buffers) belongs to that call:
         # hand it back to the context's pool, as the reference harness does after every case (litert.hpp:268-276);
         # the pool is reused in stream order, so a later call on this context may overwrite it safely
