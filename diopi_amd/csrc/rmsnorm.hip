@@ -456,7 +456,7 @@ __global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight
     const int col = blockIdx.x * kCols + c;
     double sw = 0.0, sb = 0.0;
     if (col < n2) {
-        constexpr int kBatch = 8;  // loads of a batch are independent and in flight together
+        constexpr int kBatch = 16;  // loads of a batch are independent and in flight together: 256 partial rows are one round trip
         for (int p0 = slice; p0 < numParts; p0 += kSlices * kBatch) {
             ColAcc vw[kBatch], vb[kBatch];
 #pragma unroll

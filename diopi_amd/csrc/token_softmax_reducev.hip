@@ -350,17 +350,10 @@ __global__ __launch_bounds__(kRvThreads) void softmaxReduceVMerge(T* __restrict_
     const int qh = idx / a.D, d = idx % a.D;
     const float* ml = sp.partMl + (static_cast<int64_t>(i) * sp.splits * a.H + qh) * 2;
     const float* pa = sp.partAcc + (static_cast<int64_t>(i) * sp.splits * a.H + qh) * a.D + d;
-    // ranges are visited in batches of 8 so that the loads of a batch are all in flight together
+    // One pass over the ranges, in batches of 8 whose loads are all in flight together (a sequence of up to 8 ranges costs
+    // one memory round trip): the running maximum moves from batch to batch and the sums collected so far are rescaled.
     constexpr int kBatch = 8;
-    float m = -INFINITY;
-    for (int j0 = 0; j0 < ns; j0 += kBatch) {
-        float mj[kBatch];
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) mj[u] = (j0 + u < ns) ? ml[static_cast<int64_t>(j0 + u) * a.H * 2] : -INFINITY;
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) m = fmaxf(m, mj[u]);
-    }
-    float num = 0.f, den = 0.f;
+    float m = -INFINITY, num = 0.f, den = 0.f;
     for (int j0 = 0; j0 < ns; j0 += kBatch) {
         float mj[kBatch], lj[kBatch], aj[kBatch];
 #pragma unroll
@@ -370,12 +363,19 @@ __global__ __launch_bounds__(kRvThreads) void softmaxReduceVMerge(T* __restrict_
             lj[u] = ok ? ml[static_cast<int64_t>(j0 + u) * a.H * 2 + 1] : 0.f;
             aj[u] = ok ? pa[static_cast<int64_t>(j0 + u) * a.H * a.D] : 0.f;
         }
+        float mNew = m;
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) mNew = fmaxf(mNew, mj[u]);
+        const float keep = (m == -INFINITY) ? 0.f : __expf(m - mNew);
+        num *= keep;
+        den *= keep;
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
-            const float w = (mj[u] == -INFINITY) ? 0.f : __expf(mj[u] - m);
+            const float w = (mj[u] == -INFINITY) ? 0.f : __expf(mj[u] - mNew);
             num += w * aj[u];
             den += w * lj[u];
         }
+        m = mNew;
     }
     out[(static_cast<int64_t>(i) * a.H + qh) * a.D + d] = static_cast<T>(num / den);
 }
