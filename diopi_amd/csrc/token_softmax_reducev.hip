@@ -9,8 +9,9 @@
 // other_kv_index is ignored, as in the reference.
 //
 // Kernel shape (16-bit types, D == 128, G <= 16): a split-K ("flash decoding") pass on the matrix cores followed
-// by a small merge.  A wave owns (kv head, token range, sequence); it never synchronises with other waves.  The
-// range's (max, denominator, accumulator) triple goes to context-owned scratch and a merge kernel combines the
+// by a small merge.  A work-group owns (kv head, token range, sequence); its four waves take the range's 128-token
+// sub-tiles in turn, never meet at a barrier while they stream, and combine their (max, denominator, accumulator)
+// triples in LDS at the end.  The range's triple goes to context-owned scratch and a merge kernel combines the
 // ranges of a sequence; a sequence that fits one range is finished in place and skips the scratch round trip.
 // V bytes are read exactly once.  Nothing on the host depends on the sequence lengths.
 // Everything else (fp32 / fp64, other head sizes, G > 16) takes a shape-agnostic kernel.
@@ -33,13 +34,14 @@ struct SplitArgs {
     float* partMl;   // [batch, splits, H, 2]  (running max, denominator)
     int splits;      // ranges per sequence the scratch is sized for
     int TT;          // tokens per range (multiple of kSub)
+    int headsPerGroup;  // kv heads a work-group streams side by side: 1, 2 or 4 (its waves are heads x sub-tile phases)
 };
 
 // Matrix-core kernel (16-bit types, D == 128, any G <= 16): per kv head the weighted sum is the small product
 //   out[g, d] += P[g, t] . V[t, d]      on v_mfma_f32_16x16x32 (16 query heads x 16 dims x 32 tokens),
 // so the vector-ALU work per V byte does not grow with G.
-// A wave owns (kv head, token range, sequence), i.e. the G query heads of its kv head, and walks the range in
-// sub-tiles of 128 tokens without ever meeting another wave at a barrier:
+// A wave works for the G query heads of its work-group's kv head and walks its share of the range (every fourth
+// sub-tile of 128 tokens) without meeting another wave before the final hand-over:
 //   * logits of the sub-tile: per query head two coalesced loads (lane = token), prefetched one sub-tile ahead
 //     (tokens past the range alias its last one and become -inf by a select): no load sits inside a branch, so all of
 //     them stay in flight until the next sub-tile's softmax;
@@ -54,9 +56,9 @@ struct SplitArgs {
 //     so the wave always has rows in flight;
 //   * the A operand (8 consecutive tokens of query head l % 16) is one 16-byte read of the probability tile;
 //   * C holds out[4 * (l / 16) + r][8 * (l % 16) + e] in acc[e][r]: a lane ends up with 8 consecutive dims of up to
-//     four query heads, which are stored directly; accumulator rows are rescaled only when some head's maximum
-//     moved (a wave-uniform test).
+//     four query heads; accumulator rows are rescaled only when some head's maximum moved (a wave-uniform test).
 constexpr int kTilePitch = kSub + 8;  // elements per probability row; 272 bytes
+constexpr int kMergePitch = kD + 4;   // floats per query head in the hand-over of a work-group's waves: 128 sums, maximum, denominator
 
 // LDS that only one wave touches needs no barrier (the LDS executes a wave's operations in order), but the compiler
 // must not move accesses of different types across the hand-over points.
@@ -75,7 +77,7 @@ __device__ __forceinline__ float waveSumUniform(float v) {
     return (laneValue(v, 0) + laneValue(v, 16)) + (laneValue(v, 32) + laneValue(v, 48));
 }
 
-template <typename T, int GC, int HPW>
+template <typename T, int GC>
 __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
                                                                     SplitArgs sp) {
     using Ops = Mfma16<T>;
@@ -83,8 +85,9 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     __shared__ __attribute__((aligned(16))) T sP[kRvWaves][GC * kTilePitch];
     __shared__ __attribute__((aligned(16))) int32_t sSlotW[kRvWaves][kSub];
     __shared__ __attribute__((aligned(16))) float sStat[kRvWaves][16];
+    __shared__ __attribute__((aligned(16))) float sMerge[kRvWaves][GC][kMergePitch];  // per wave and query head: 128 sums, maximum, denominator
 
-    // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
+    // x runs over kv heads (neighbouring work-groups read neighbouring 256-byte pieces of the same cache rows at the same
     // time), y over sequences, z over token ranges, with the sequence rotated by the range index so that consecutive
     // work-groups (dealt round-robin to the 8 XCDs) mix ranges of different sequences: with ragged lengths no XCD is
     // left with only the sparse late ranges
@@ -92,44 +95,48 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
     const int64_t t0 = static_cast<int64_t>(blockIdx.z) * sp.TT;
+    const int HG = sp.headsPerGroup;
+    const int phases = kRvWaves / HG;  // waves that share a kv head take the sub-tiles in turn
+    const int waveId = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int hkRaw = blockIdx.x * HG + waveId % HG;
+    const bool headLive = hkRaw < a.Hkv;
+    const int hk = headLive ? hkRaw : a.Hkv - 1;  // a wave past the last kv head streams nothing and writes nothing
+    const int phase = waveId / HG;
     if (t0 >= L) {
         // a sequence without tokens: the reference's product over an empty inner dimension gives zeros
         // (functions_lightllm.cpp:98-104); the work-groups of range 0 write them
-        if (L <= 0 && blockIdx.z == 0) {
-            const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
-            const int hk0 = (blockIdx.x * kRvWaves + w) * HPW;
-            const int rows = (hk0 < a.Hkv) ? ((a.Hkv - hk0 < HPW ? a.Hkv - hk0 : HPW) * a.G) : 0;
+        if (L <= 0 && blockIdx.z == 0 && phase == 0 && headLive) {
+            const int l = threadIdx.x % kWave;
             Pack16<T> z;
             z.raw = u32x4{0u, 0u, 0u, 0u};
-            for (int g = l / 16; g < rows; g += 4) storePack(out + (static_cast<int64_t>(i) * a.H + hk0 * a.G + g) * kD + (l % 16) * 8, z);
+            for (int g = l / 16; g < a.G; g += 4) storePack(out + (static_cast<int64_t>(i) * a.H + hk * a.G + g) * kD + (l % 16) * 8, z);
         }
         return;
     }
+    // The range of the work-group, cut into sub-tiles of 128 tokens that the waves of a kv head take in turn (phase p the
+    // sub-tiles p, p + phases, ...): several waves stream one (sequence, kv head, range) that many times as fast as one would,
+    // and what leaves the work-group is one partial result per kv head.
     const int64_t tEnd = (t0 + sp.TT < L) ? t0 + sp.TT : L;
-    const int nTokR = static_cast<int>(tEnd - t0);
-    const int nSub = (nTokR + kSub - 1) / kSub;
+    const int nTokR = static_cast<int>(tEnd - t0);             // tokens of the work-group's range
+    const int nSubAll = (nTokR + kSub - 1) / kSub;
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
     const int64_t locBase = static_cast<int64_t>(i) * a.bLocStride + (a.maxInputLen - L) + t0;
     const int tid = threadIdx.x;
     const int lane = tid % kWave;
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    // HPW == 1: the wave streams one kv head; lane group q takes tokens 8q .. 8q+7 of every 32-token step.
-    // HPW == 4: the wave streams four adjacent kv heads (1 KiB contiguous per token, which the memory system likes
-    //           better); lane group q takes head q and the same 8 tokens per step as the other groups.  The four
-    //           heads share the products through a block-diagonal A operand: row m only carries probabilities in the
-    //           lane group of its own kv head, zeros elsewhere.
+    const int wave = waveId;
+    const int nSub = (headLive && phase < nSubAll) ? (nSubAll - phase + phases - 1) / phases : 0;  // sub-tiles of this wave
+    auto subOff = [&](int sub) { return (sub * phases + phase) * kSub; };                           // first token of its sub-tile `sub`
+    // lane group q takes tokens 8q .. 8q+7 of every 32-token step
     const int q = lane / 16;
     const int c = lane % 16;  // 16-byte packet of the row segment; also the row (query head) of the A operand
     const int G = a.G;
-    const int R = HPW * G;    // query heads (rows of the A operand) of this wave, <= GC
-    const int hk = (blockIdx.x * kRvWaves + wave) * HPW;  // first kv head of the wave
-    if (hk >= a.Hkv) return;
-    constexpr int kStep = HPW == 1 ? 32 : 8;  // tokens per step
+    const int R = G;          // query heads (rows of the A operand) of this wave, <= GC
+    constexpr int kStep = 32;  // tokens per step
     const int64_t rowStride = static_cast<int64_t>(a.Hkv) * kD;
     T* tile = &sP[wave][0];
     int32_t* slotW = &sSlotW[wave][0];
     float* statW = &sStat[wave][0];
-    const T* vHead = v + (hk + (HPW == 1 ? 0 : q)) * kD + c * 8;
+    const T* vHead = v + hk * kD + c * 8;
     const int64_t colBase = start + t0;
     // tokens of the range whose logits exist: the range may stick out of the logits columns only on invalid input
     int nLogit = 0;
@@ -150,7 +157,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         for (int g = 0; g < GC; ++g) {
 #pragma unroll
             for (int k = 0; k < 2; ++k) {
-                const int t = sub * kSub + 64 * k + lane;
+                const int t = subOff(sub) + 64 * k + lane;
                 const int tc = t < nLogit ? t : nLogit - 1;
                 const unsigned short raw =
                     __builtin_amdgcn_raw_buffer_load_b16(xBuf, (g < R ? g : 0) * xRowBytes + tc * static_cast<int>(sizeof(T)), 0, 0);
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     auto loadSlots = [&](int sub) {
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
-            int t = sub * kSub + 64 * k + lane;
+            int t = subOff(sub) + 64 * k + lane;
             t = t < nTokR ? t : nTokR - 1;  // tokens past the end alias the last valid one (their probability is zero)
             slotLo[k] = __builtin_amdgcn_raw_buffer_load_b32(locBuf, t * locElem, 0, 0);
             slotHi[k] = __builtin_amdgcn_raw_buffer_load_b32(locBuf, t * locElem, a.loc64 ? 4 : 0, 0);
@@ -189,7 +196,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     // two sets of 8 rows per lane: while the products of one step consume a set, the rows of the next step are in flight
     u32x4 rowsA[8], rowsB[8];
     auto issueV = [&](int step, u32x4 (&rows)[8]) {
-        const int first = HPW == 1 ? 32 * step + 8 * q : 8 * step;
+        const int first = 32 * step + 8 * q;
         const u32x4 s0 = *reinterpret_cast<const u32x4*>(slotW + first);
         const u32x4 s1 = *reinterpret_cast<const u32x4*>(slotW + first + 4);
 #pragma unroll
@@ -200,17 +207,19 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     };
     static_assert((kSub / kStep) % 2 == 0, "a set of row registers keeps its parity from one sub-tile to the next");
     auto stepsOf = [&](int sub) {
-        const int n = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
+        const int n = (nTokR - subOff(sub) < kSub) ? nTokR - subOff(sub) : kSub;
         return (n + kStep - 1) / kStep;
     };
 
     // the first logits are requested before the first rows: the softmax of sub-tile 0 then only waits for them, as
     // the softmax of every later sub-tile does, while rows are in flight
-    loadSlots(0);
-    loadLogits(0);
-    storeSlots();
-    issueV(0, rowsA);
-    if (stepsOf(0) > 1) issueV(1, rowsB);
+    if (nSub > 0) {  // a wave without sub-tiles (a short range) only takes part in the hand-over below
+        loadSlots(0);
+        loadLogits(0);
+        storeSlots();
+        issueV(0, rowsA);
+        if (stepsOf(0) > 1) issueV(1, rowsB);
+    }
 
     f32x4 acc[8];
 #pragma unroll
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     }
 
     for (int sub = 0; sub < nSub; ++sub) {
-        const int nTok = (nTokR - sub * kSub < kSub) ? nTokR - sub * kSub : kSub;
+        const int nTok = (nTokR - subOff(sub) < kSub) ? nTokR - subOff(sub) : kSub;
         const int nSteps = (nTok + kStep - 1) / kStep;
         // ---- softmax of the sub-tile ----
         waveLdsFence();
@@ -255,9 +264,9 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
             for (int e = 0; e < 8; ++e) acc[e] *= al;
         }
         // ---- P . V on the matrix cores ----
-        // A operand: row c, the 8 tokens of this lane group's k slots; rows of other kv heads contribute zeros
-        const bool rowLive = HPW == 1 ? c < G : (c < R && c / G == q);
-        const T* pRow = tile + (c < R ? c : 0) * kTilePitch + (HPW == 1 ? 8 * q : 0);
+        // A operand: row c, the 8 tokens of this lane group's k slots; rows past the last query head are zeros
+        const bool rowLive = c < G;
+        const T* pRow = tile + (c < R ? c : 0) * kTilePitch + 8 * q;
         const int nStepsNext = (sub + 1 < nSub) ? stepsOf(sub + 1) : 0;
         auto pvStep = [&](int s, u32x4 (&rowsV)[8]) {
             union {
@@ -300,39 +309,57 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         }
     }
 
-    // ---- hand the denominators to the lanes that hold the matching accumulator rows, then store ----
-    waveLdsFence();
+    // ---- the waves of the work-group hand their (maximum, denominator, sums) over in LDS; all threads combine them ----
+    {
+        float* mine = &sMerge[wave][0][0];
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-        if (lane == 0) statW[g] = lRun[g];
+        for (int r = 0; r < 4; ++r) {
+            const int g = 4 * q + r;
+            if (g < G) {
+                *reinterpret_cast<f32x4*>(mine + g * kMergePitch + 8 * c) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+                *reinterpret_cast<f32x4*>(mine + g * kMergePitch + 8 * c + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+            if (lane == g && g < G) {
+                mine[g * kMergePitch + kD] = mRun[g];
+                mine[g * kMergePitch + kD + 1] = lRun[g];
+            }
+        }
     }
-    waveLdsFence();
+    __syncthreads();
     const bool single = L <= sp.TT;  // the whole sequence lives in this range
-    const int64_t split = blockIdx.z;
-    if (!single && lane < R) {
-        // lane g publishes (max, denominator) of query head g
-        float mg = -INFINITY;
+    for (int idx = tid; idx < HG * G * kD; idx += kRvThreads) {
+        const int hl = idx / (G * kD);  // kv head of the work-group
+        const int g = idx / kD % G, d = idx % kD;
+        if (blockIdx.x * HG + hl >= a.Hkv) break;
+        float mw[kRvWaves];
+        float m = -INFINITY;
 #pragma unroll
-        for (int g = 0; g < GC; ++g) mg = (lane == g) ? mRun[g] : mg;
-        float* ml = sp.partMl + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + hk * G + lane) * 2;
-        ml[0] = mg;
-        ml[1] = statW[lane];
-    }
+        for (int p = 0; p < kRvWaves; ++p) {
+            mw[p] = p < phases ? sMerge[p * HG + hl][g][kD] : -INFINITY;
+            m = fmaxf(m, mw[p]);
+        }
+        float num = 0.f, den = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int g = 4 * q + r;
-        if (g >= R) continue;
-        const int qh = hk * G + g;
+        for (int p = 0; p < kRvWaves; ++p) {
+            if (p < phases) {
+                const float wgt = (mw[p] == -INFINITY) ? 0.f : __expf(mw[p] - m);  // a wave without tokens has maximum -inf and weighs nothing
+                num += wgt * sMerge[p * HG + hl][g][d];
+                den += wgt * sMerge[p * HG + hl][g][kD + 1];
+            }
+        }
+        const int qh = (blockIdx.x * HG + hl) * G + g;
         if (single) {
-            const float inv = 1.f / statW[g];
-            Pack16<T> o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o.e[e] = static_cast<T>(acc[e][r] * inv);
-            storePack(out + (static_cast<int64_t>(i) * a.H + qh) * kD + c * 8, o);
+            out[(static_cast<int64_t>(i) * a.H + qh) * kD + d] = static_cast<T>(num / den);
         } else {
-            float* dst = sp.partAcc + ((static_cast<int64_t>(i) * sp.splits + split) * a.H + qh) * kD + c * 8;
-            *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+            const int64_t slot = (static_cast<int64_t>(i) * sp.splits + blockIdx.z) * a.H + qh;
+            sp.partAcc[slot * kD + d] = num;
+            if (d == 0) {
+                sp.partMl[slot * 2] = m;
+                sp.partMl[slot * 2 + 1] = den;
+            }
         }
     }
 }
@@ -447,13 +474,15 @@ __global__ __launch_bounds__(kRvThreads) void softmaxReduceVGeneric(T* __restric
 template <typename T>
 diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out, const void* logits, const void* v, const DecodeArgs& a) {
     SplitArgs sp;
-    // tokens per range: the fp32 partial (G*D*4 bytes per kv head) against the V bytes it summarises (TT*D*2): about
-    // 1.5 % at TT = 128*G; shorter ranges balance ragged batches better, longer ones amortise the pipeline start
-    // (measured with one query head per kv head, 64 sequences of 512..2048 tokens: 256 and 384 tokens per range are
-    // 1 % faster than 512, 1024 is 7 % slower)
-    int TT = 128 * a.G;
-    if (TT < 256) TT = 256;
-    if (TT > 2048) TT = 2048;
+    // tokens per work-group range.  What leaves a range is an fp32 partial of G*(D+2)*4 bytes per kv head, and those
+    // writes are dear next to the row gather (8.5 MB of them cost 10 us of 111 at 64 sequences of 512..2048 tokens and
+    // one query head per kv head; 19 MB cost 27 us of 236 at 128 sequences of 1024..8192 tokens and 8 query heads per
+    // kv head): ranges are long, and the four waves of a work-group share one so that it still streams quickly.
+    // Measured: ranges of 2560..5120 tokens 227-229 us at the second shape (6144: 231, 8192: 243 - too few work-groups),
+    // 768..4096 tokens 107.5-110 us at the first.
+    int TT = 512 * a.G;
+    if (TT < 2048) TT = 2048;
+    if (TT > 8192) TT = 8192;
     TT = envInt("DIOPI_ROCM_REDUCEV_TT", TT);
     TT = static_cast<int>(ceilDiv(TT, kSub)) * kSub;
     sp.TT = TT;
@@ -470,32 +499,25 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     }
     ROCM_CHECK(a.batch <= 65535, "batch %d exceeds the launch limit of 65535 sequences", a.batch);
     ROCM_CHECK(sp.splits <= 65535, "max_input_len %d needs more than 65535 ranges of %d tokens", a.maxInputLen, TT);
-    // four adjacent kv heads per wave (1 KiB contiguous per token) when their query heads fit the 16 rows of a product
-    const bool quad = a.G <= 4 && a.Hkv % 4 == 0 && envInt("DIOPI_ROCM_REDUCEV_QUAD", 0) != 0;
-    const int hpw = quad ? 4 : 1;
-    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, kRvWaves * hpw)), static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits));
-#define ROCM_RVW_CASE(GC, HPW)                                                                                                                   \
-    hipLaunchKernelGGL((softmaxReduceVWave<T, GC, HPW>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
+    // kv heads per work-group: 1, 2 or 4 of the four waves' worth (the others are sub-tile phases of the same head); one
+    // head per work-group measured best or equal at both shapes above (2 and 4 heads: up to 8 % slower with grouped heads)
+    int HG = envInt("DIOPI_ROCM_REDUCEV_HEADS", 1);
+    if (HG != 1 && HG != 2 && HG != 4) HG = 1;
+    sp.headsPerGroup = HG;
+    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HG)), static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits));
+#define ROCM_RVW_CASE(GC)                                                                                                                   \
+    hipLaunchKernelGGL((softmaxReduceVWave<T, GC>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
                        static_cast<const T*>(v), a, sp)
-    const int rows = hpw * a.G;
-    if (quad) {
-        if (rows <= 4) {
-            ROCM_RVW_CASE(4, 4);
-        } else if (rows <= 8) {
-            ROCM_RVW_CASE(8, 4);
-        } else {
-            ROCM_RVW_CASE(16, 4);
-        }
-    } else if (rows <= 1) {
-        ROCM_RVW_CASE(1, 1);
-    } else if (rows <= 2) {
-        ROCM_RVW_CASE(2, 1);
-    } else if (rows <= 4) {
-        ROCM_RVW_CASE(4, 1);
-    } else if (rows <= 8) {
-        ROCM_RVW_CASE(8, 1);
+    if (a.G <= 1) {
+        ROCM_RVW_CASE(1);
+    } else if (a.G <= 2) {
+        ROCM_RVW_CASE(2);
+    } else if (a.G <= 4) {
+        ROCM_RVW_CASE(4);
+    } else if (a.G <= 8) {
+        ROCM_RVW_CASE(8);
     } else {
-        ROCM_RVW_CASE(16, 1);
+        ROCM_RVW_CASE(16);
     }
 #undef ROCM_RVW_CASE
     ROCM_LAUNCH_CHECK();

@@ -581,9 +581,9 @@ def test_decode_sequences_sharing_cache_rows(dtype, Hq, Hkv):
 
 def test_decode_range_length_follows_each_call_not_the_first_one():
     """The range length of the split decode kernel depends on the head grouping of the call at hand.  The scratch a call
-    asks for shows it: B * ceil(max_len / range) * H * (D + 2) * 4 bytes with range = max(256, 128 * G)."""
+    asks for shows it: B * ceil(max_len / range) * H * (D + 2) * 4 bytes with range = max(2048, 512 * G)."""
     g = gen(570)
-    D, slots, maxlen, B = 128, 4096, 2048, 2
+    D, slots, maxlen, B = 128, 8192, 8192, 2
 
     def scratch_of(Hq, Hkv):
         ctx = rt.Context(own_stream=True)
@@ -601,7 +601,7 @@ def test_decode_range_length_follows_each_call_not_the_first_one():
         return peak
 
     def expected(Hq, Hkv):
-        rng_len = max(256, 128 * (Hq // Hkv))
+        rng_len = max(2048, 512 * (Hq // Hkv))
         return B * math.ceil(maxlen / rng_len) * Hq * (D + 2) * 4
 
     for Hq, Hkv in ((4, 4), (8, 1), (4, 4), (8, 2)):  # ungrouped first, then grouped, and back
