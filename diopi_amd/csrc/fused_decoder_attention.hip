@@ -27,7 +27,8 @@
 //                    straight into the cache.  HBM-bound on the weights.  With few heads and rows the hidden dimension is
 //                    also cut across work-groups (up to one work-group per compute unit in all); their fp32 sums then go
 //                    through the workspace and fusedQkvFinish adds them and does the bias, rotation and stores.
-//   fusedDecodeAttn  a wave owns (batch row, kv head, range of cached tokens): per 32 tokens 8 K loads that arrive in
+//   fusedDecodeAttn  a work-group owns (batch row, kv head, range of 512 cached tokens) and its four waves take the range's
+//                    128-token chunks in turn, meeting only for a final hand-over in LDS; per 32 tokens 8 K loads that arrive in
 //                    the B-operand layout of q.k^T (16 lanes x 16-byte pieces of 16 consecutive cache rows), online
 //                    softmax on the 16 x 32 scores (row maxima and sums by DPP row reductions), probabilities through a
 //                    wave-private LDS tile into the A-operand layout, 8 V loads permuted as above for P.V.  The scores
@@ -285,18 +286,30 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
     __shared__ __attribute__((aligned(16))) T sP[kAttnWaves][16 * kProbPitch];
+    __shared__ __attribute__((aligned(16))) float sMerge[kAttnWaves][16][kFD + 4];  // per wave and query head: 128 sums, maximum, denominator
     const int b = blockIdx.y;
     const int split = blockIdx.z;
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int hk = blockIdx.x * kAttnWaves + wave;
-    if (hk >= a.Hkv || rowFinished(a, b)) return;  // waves never meet at a barrier
+    const int hk = blockIdx.x;  // the kv head of this work-group
+    if (rowFinished(a, b)) return;
     const int64_t L = rowLength(a, b);
     const int nWin = static_cast<int>(L + 1 < a.maxSeq ? L + 1 : a.maxSeq);  // tokens in the window, the new one last
     const int t0 = split * sp.TT;
     if (t0 >= nWin) return;
-    const int nTok = nWin - t0 < sp.TT ? nWin - t0 : sp.TT;
-    const int nSteps = (nTok + kAttnStep - 1) / kAttnStep;
+    // The range of the work-group is cut into chunks of 128 tokens that its four waves take in turn (wave w the chunks
+    // w, w + 4, ...): a (row, kv head) streams four times as fast as one wave would, and what leaves the work-group is one
+    // result.  Local token i of a wave is token (4 * (i / 128) + w) * 128 + i % 128 of the range.
+    constexpr int kChunk = 4 * kAttnStep;
+    const int nTok = nWin - t0 < sp.TT ? nWin - t0 : sp.TT;  // tokens of the range
+    const int nChunks = (nTok + kChunk - 1) / kChunk;
+    const int myChunks = wave < nChunks ? (nChunks - wave + kAttnWaves - 1) / kAttnWaves : 0;
+    int nSteps = 0;
+    if (myChunks > 0) {
+        const int lastStart = ((myChunks - 1) * kAttnWaves + wave) * kChunk;  // first token of this wave's last chunk
+        const int lastTok = nTok - lastStart < kChunk ? nTok - lastStart : kChunk;
+        nSteps = (myChunks - 1) * (kChunk / kAttnStep) + (lastTok + kAttnStep - 1) / kAttnStep;
+    }
     const int firstPos = static_cast<int>((L + 1 - nWin) % a.maxSeq);  // cache row of the window's first token
     const int g4 = lane / 16;
     const int c = lane % 16;
@@ -305,9 +318,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
     const T* kHead = kCache + headOff + 8 * g4;  // + row * D + 32 s: 8 dims of k block g4
     const T* vHead = vCache + headOff + 8 * c;   // + row * D: packet c of a row
     T* tile = sP[wave];
-    // cache row of token i of the range; tokens past the range repeat its last one (their scores become -inf)
+    // token of the range behind local token i of this wave
+    auto tokenOf = [&](int i) { return ((i / kChunk) * kAttnWaves + wave) * kChunk + i % kChunk; };
+    // its cache row; tokens past the range repeat the range's last one (their scores become -inf)
     auto rowOf = [&](int i) {
-        int p = firstPos + t0 + (i < nTok ? i : nTok - 1);
+        const int t = tokenOf(i);
+        int p = firstPos + t0 + (t < nTok ? t : nTok - 1);
         p = p >= a.maxSeq ? p - a.maxSeq : p;
         return static_cast<int64_t>(p) * kFD;
     };
@@ -336,8 +352,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
 #pragma unroll
         for (int r = 0; r < 8; ++r) vb[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + rowOf(kAttnStep * st + 8 * g4 + r)));
     };
-    issueK(0);
-    issueV(0);
+    if (nSteps > 0) {  // a wave without chunks (a short range) only takes part in the hand-over below
+        issueK(0);
+        issueV(0);
+    }
 
     f32x4 acc[8];
 #pragma unroll
@@ -372,7 +390,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
         bool moved = false;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool ok0 = kAttnStep * st + c < nTok, ok1 = kAttnStep * st + 16 + c < nTok;
+            const bool ok0 = tokenOf(kAttnStep * st + c) < nTok, ok1 = tokenOf(kAttnStep * st + 16 + c) < nTok;
             const float s0 = ok0 ? sc[0][r] * scale : -INFINITY;
             const float s1 = ok1 ? sc[1][r] * scale : -INFINITY;
             const float mNew = fmaxf(mRun[r], rowMax16(fmaxf(s0, s1)));  // finite: every step holds a token of the range
@@ -417,27 +435,49 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
         issueV(st + 1);
     }
 
-    // ---- acc[e][r] is dim 8c + e of query head 4 g4 + r
-    const bool single = nWin <= sp.TT;
+    // ---- acc[e][r] is dim 8c + e of query head 4 g4 + r: the waves hand their (maximum, denominator, sums) over in LDS
+    {
+        float* mine = &sMerge[wave][0][0];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int g = 4 * g4 + r;
-        if (g >= G) continue;
+        for (int r = 0; r < 4; ++r) {
+            const int g = 4 * g4 + r;
+            if (g < G) {
+                *reinterpret_cast<f32x4*>(mine + g * (kFD + 4) + 8 * c) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+                *reinterpret_cast<f32x4*>(mine + g * (kFD + 4) + 8 * c + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+                if (c == 0) {
+                    mine[g * (kFD + 4) + kFD] = mRun[r];
+                    mine[g * (kFD + 4) + kFD + 1] = lRun[r];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const bool single = nWin <= sp.TT;
+    for (int idx = threadIdx.x; idx < G * kFD; idx += kAttnThreads) {
+        const int g = idx / kFD, d = idx % kFD;
+        float mw[kAttnWaves];
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            mw[w] = sMerge[w][g][kFD];
+            m = fmaxf(m, mw[w]);
+        }
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            const float wgt = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - m);  // a wave without tokens weighs nothing
+            num += wgt * sMerge[w][g][d];
+            den += wgt * sMerge[w][g][kFD + 1];
+        }
         const int qh = hk * G + g;
         if (single) {
-            const float inv = 1.0f / (lRun[r] + 1e-6f);
-            Pack16<T> o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o.e[e] = static_cast<T>(acc[e][r] * inv);
-            storePack(out + static_cast<int64_t>(b) * a.hidden + qh * kFD + 8 * c, o);
+            out[static_cast<int64_t>(b) * a.hidden + qh * kFD + d] = static_cast<T>(num / (den + 1e-6f));
         } else {
             const int64_t slot = (static_cast<int64_t>(b) * sp.splits + split) * a.H + qh;
-            float* dst = sp.partAcc + slot * kFD + 8 * c;
-            *reinterpret_cast<f32x4*>(dst) = f32x4{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
-            if (c == 0) {
-                sp.partMl[slot * 2] = mRun[r];
-                sp.partMl[slot * 2 + 1] = lRun[r];
+            sp.partAcc[slot * kFD + d] = num;
+            if (d == 0) {
+                sp.partMl[slot * 2] = m;
+                sp.partMl[slot * 2 + 1] = den;
             }
         }
     }
@@ -490,7 +530,7 @@ diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const v
                            static_cast<const T*>(bias), a, projParts);
         ROCM_LAUNCH_CHECK();
     }
-    const dim3 agrid(static_cast<unsigned>(ceilDiv(a.Hkv, kAttnWaves)), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
+    const dim3 agrid(static_cast<unsigned>(a.Hkv), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
     hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), 0, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
                        static_cast<const T*>(vCache), a, sp);
     ROCM_LAUNCH_CHECK();
@@ -575,9 +615,11 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
                      static_cast<long long>(hidden));
         return diopiNoImplement;
     }
-    // ranges of the attention kernel: 256 cached tokens each when kv heads are plentiful, the workspace sized for max_seq_len
+    // ranges of the attention kernel: 512 cached tokens per work-group (its four waves share them), the workspace sized for
+    // max_seq_len.  Measured at 64 rows of 511..2047 tokens, 32 kv heads: 256..1024 tokens per range within 1.5 us of each
+    // other, 2048 (no partials, no merge launch) 7 us slower: rows of unequal length then leave the last work-groups alone
     AttnSplit sp;
-    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 256);
+    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 512);
     sp.TT = static_cast<int>(ceilDiv(sp.TT, kAttnStep)) * kAttnStep;
     sp.splits = static_cast<int>(ceilDiv(max_seq_len, sp.TT));
     sp.partAcc = nullptr;
