@@ -16,17 +16,17 @@
 // Open in the prose, fixed here: the rotary pairing (2), a circular cache window once L reaches max_seq_len (3, 4),
 // where the output lands when H*D < hidden_units (5), and that finished rows are left untouched everywhere.
 //
-// Three kernels (four when the projection's hidden dimension is split), all on the context's stream:
-//   fusedQkvHead     one work-group per head of the projection (128 output columns) and 64 batch rows.  The weight
-//                    panel [hidden, 128] goes through 8 waves = 4 quarters of the hidden dimension x 2 halves of the batch
-//                    rows.  A lane loads 8 consecutive weight rows (16 bytes = 8 columns each); pairs of rows
-//                    interleaved with two byte permutes become the B operands of v_mfma_f32_16x16x32 for the lane's 8
-//                    columns and serve two products (two blocks of 16 batch rows, whose A operands are 16 bytes of a
-//                    hidden-state row each).  The quarters meet in LDS (fp32), and
-//                    the same work-group adds the bias, rotates, and writes the head: q to the workspace, k and v
-//                    straight into the cache.  HBM-bound on the weights.  With few heads and rows the hidden dimension is
-//                    also cut across work-groups (up to one work-group per compute unit in all); their fp32 sums then go
-//                    through the workspace and fusedQkvFinish adds them and does the bias, rotation and stores.
+// Four kernels, all on the context's stream:
+//   fusedQkvPart     the projection, HBM-bound on the weights.  Its units (a 32-row step of the hidden dimension of one
+//                    128-column head) go in equal runs to one work-group per compute unit: a compute unit draws a bounded
+//                    share of the memory bandwidth, so all of them have to pull, whatever the number of heads.  The four
+//                    waves of a work-group split a run's steps and each covers all 64 batch rows: a lane loads 8
+//                    consecutive weight rows (16 bytes = 8 columns each); pairs of rows interleaved with two byte permutes
+//                    become the B operands of v_mfma_f32_16x16x32 for the lane's 8 columns and serve four products (four
+//                    blocks of 16 batch rows, whose A operands are 16 bytes of a hidden-state row each).  The waves meet
+//                    in LDS (fp32, 132 KiB) and the work-group writes one fp32 partial tile per head its run touched.
+//   fusedQkvFinish   adds the partial tiles of a head, rounds, adds the bias, rotates, and writes the head: q to the
+//                    workspace, k and v straight into the cache.
 //   fusedDecodeAttn  a work-group owns (batch row, kv head, range of 512 cached tokens) and its four waves take the range's
 //                    128-token chunks in turn, meeting only for a final hand-over in LDS; per 32 tokens 8 K loads that arrive in
 //                    the B-operand layout of q.k^T (16 lanes x 16-byte pieces of 16 consecutive cache rows), online
@@ -36,6 +36,7 @@
 //   fusedDecodeMerge combines the ranges of a row (skipped when the window fits one range).
 #include <diopi/functions_lmdeploy.h>
 
+#include <algorithm>
 #include <cmath>
 
 #include "common.hpp"
@@ -45,9 +46,10 @@ namespace rocm {
 namespace {
 
 constexpr int kFD = 128;          // head size of the fast path
-constexpr int kProjThreads = 512;
-constexpr int kProjRB = 2;         // blocks of 16 batch rows per wave
-constexpr int kProjSlabs = kProjThreads / kWave / 2;  // slabs of the hidden dimension: waves = 2 row halves x slabs
+constexpr int kProjThreads = 256;
+constexpr int kProjWaves = kProjThreads / kWave;  // each with its own steps of the hidden dimension
+constexpr int kProjRB = 4;         // blocks of 16 batch rows per wave: all 64 rows of the work-group
+constexpr int kProjDepth = 2;      // steps of a wave in flight
 constexpr int kProjRows = 64;     // batch rows per work-group of the projection
 constexpr int kProjPitch = kFD + 4;  // floats per row of a partial tile: rows 4 apart are 16 banks apart
 constexpr int kAttnThreads = 256;
@@ -113,89 +115,119 @@ __device__ __forceinline__ void finishPair(T* __restrict__ qOut, T* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
+// How the projection is cut: a unit is one 32-row step of the hidden dimension of one 128-column head; the units, head
+// after head, are dealt out in equal runs to as many work-groups as the device has compute units (a compute unit draws
+// a bounded share of the memory bandwidth, so every one of them has to pull).  A run may end inside a head and go on in
+// the next one: a work-group then writes one partial tile per head it touched, and a head gets its partial tiles from
+// the work-groups first(t) .. last(t), in slots 0 .. last(t) - first(t).
+struct ProjPlan {
+    int tiles;         // heads of the projection: H + 2 Hkv
+    int stepsPerTile;  // hidden / 32
+    int unitsPerWg;
+    int slots;         // partial tiles kept per head (the most any head gets)
+};
+__host__ __device__ __forceinline__ int projFirstWg(const ProjPlan& pl, int tile) { return tile * pl.stepsPerTile / pl.unitsPerWg; }
+__host__ __device__ __forceinline__ int projLastWg(const ProjPlan& pl, int tile) { return ((tile + 1) * pl.stepsPerTile - 1) / pl.unitsPerWg; }
+
 template <typename T>
-__global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, float* __restrict__ hiddenPart,
-                                                            const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ bias, FusedArgs a) {
+__global__ __launch_bounds__(kProjThreads, 1) void fusedQkvPart(float* __restrict__ hiddenPart, const T* __restrict__ x, const T* __restrict__ w, FusedArgs a,
+                                                               ProjPlan pl) {
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
-    extern __shared__ __attribute__((aligned(16))) float part[];  // [kProjSlabs / 2][64 rows][kProjPitch]
-    const int tile = blockIdx.x;  // head of the projection: H query heads, then Hkv key heads, then Hkv value heads
+    extern __shared__ __attribute__((aligned(16))) float part[];  // [kProjWaves][64 rows][kProjPitch]
     const int rowBase = blockIdx.y * kProjRows;
-    const int N = (a.H + 2 * a.Hkv) * kFD;
+    const int N = pl.tiles * kFD;
     const int lane = threadIdx.x % kWave;
-    const int rh = (threadIdx.x / kWave) % 2;  // half of the 64 batch rows
-    const int ks = threadIdx.x / kWave / 2;    // slab of the hidden dimension
+    const int ks = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // this wave's share of a run's steps
     const int g4 = lane / 16;  // A, B: k slots 8 g4 .. + 7 of a 32-row step; C: rows 4 g4 .. + 3
     const int c = lane % 16;   // A: batch row of a block; loads: 16-byte packet (8 columns) of the panel; C: column
-    const int kPer = a.hidden / (kProjSlabs * gridDim.z);  // a multiple of 32
-    const int steps = kPer / 32;
-    const int kBeg = (blockIdx.z * kProjSlabs + ks) * kPer;
     const T* xRow[kProjRB];
 #pragma unroll
     for (int rb = 0; rb < kProjRB; ++rb) {
-        int row = rowBase + (rh * kProjRB + rb) * 16 + c;
+        int row = rowBase + rb * 16 + c;
         row = row < a.B ? row : a.B - 1;
-        xRow[rb] = x + static_cast<int64_t>(row) * a.hidden + kBeg + 8 * g4;
-    }
-    const T* wCol = w + static_cast<int64_t>(kBeg + 8 * g4) * N + tile * kFD + 8 * c;
-
-    f32x4 acc[kProjRB][8];
-#pragma unroll
-    for (int rb = 0; rb < kProjRB; ++rb) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[rb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        xRow[rb] = x + static_cast<int64_t>(row) * a.hidden + 8 * g4;
     }
     struct Step {
         u32x4 w[8];
         u32x4 x[kProjRB];
     };
-    // every step issues the same loads (past the last step the last one again), so that the wait for one step's rows
-    // leaves exactly the next step's in flight
-    auto issue = [&](int s, Step& st) {
-        const int sc = s < steps ? s : steps - 1;
+    const int units = pl.tiles * pl.stepsPerTile;
+    const int uEnd = (blockIdx.x + 1) * pl.unitsPerWg < units ? (blockIdx.x + 1) * pl.unitsPerWg : units;
+    for (int u = blockIdx.x * pl.unitsPerWg; u < uEnd;) {
+        const int tile = u / pl.stepsPerTile;
+        const int s0 = u % pl.stepsPerTile;
+        const int n = pl.stepsPerTile - s0 < uEnd - u ? pl.stepsPerTile - s0 : uEnd - u;  // steps of this head in the run
+        u += n;
+        // the waves take consecutive quarters of the n steps; a wave without steps reads some valid step and adds zeros
+        const int q = (n + kProjWaves - 1) / kProjWaves;
+        int first = s0 + ks * q;
+        const int steps = n - ks * q < 0 ? 0 : (n - ks * q < q ? n - ks * q : q);
+        first = first < pl.stepsPerTile ? first : pl.stepsPerTile - 1;
+        const T* wCol = w + static_cast<int64_t>(32 * first + 8 * g4) * N + tile * kFD + 8 * c;
+        const int xOff = 32 * first;
+
+        f32x4 acc[kProjRB][8];
 #pragma unroll
-        for (int r = 0; r < 8; ++r) st.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wCol + static_cast<int64_t>(32 * sc + r) * N));
+        for (int rb = 0; rb < kProjRB; ++rb) {
 #pragma unroll
-        for (int rb = 0; rb < kProjRB; ++rb) st.x[rb] = *reinterpret_cast<const u32x4*>(xRow[rb] + 32 * sc);
-    };
-    auto consume = [&](const Step& st) {
+            for (int e = 0; e < 8; ++e) acc[rb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        // every step issues the same loads (past the last step the last one again), so that the wait for one step's rows
+        // leaves exactly the later steps' in flight
+        auto issue = [&](int st, Step& r) {
+            int sc = st < steps ? st : steps - 1;
+            sc = sc < 0 ? 0 : sc;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            union {
-                u32x4 u;
-                Frag f;
-            } lo, hi;
+            for (int i = 0; i < 8; ++i) r.w[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wCol + static_cast<int64_t>(32 * sc + i) * N));
 #pragma unroll
-            for (int pr = 0; pr < 4; ++pr) {
-                // columns 2j and 2j+1 of this lane's packet, weight rows (2pr, 2pr+1) of the lane group
-                lo.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x05040100u);
-                hi.u[pr] = __builtin_amdgcn_perm(st.w[2 * pr + 1][j], st.w[2 * pr][j], 0x07060302u);
-            }
+            for (int rb = 0; rb < kProjRB; ++rb) r.x[rb] = *reinterpret_cast<const u32x4*>(xRow[rb] + xOff + 32 * sc);
+        };
+        // `live` is false for the steps past the last one (the ring is consumed in whole rounds): their products add zeros
+        auto consume = [&](const Step& r, bool live) {
 #pragma unroll
-            for (int rb = 0; rb < kProjRB; ++rb) {
+            for (int j = 0; j < 4; ++j) {
                 union {
                     u32x4 u;
                     Frag f;
-                } pa;
-                pa.u = st.x[rb];
-                acc[rb][2 * j] = Ops::mma(pa.f, lo.f, acc[rb][2 * j]);
-                acc[rb][2 * j + 1] = Ops::mma(pa.f, hi.f, acc[rb][2 * j + 1]);
+                } lo, hi;
+#pragma unroll
+                for (int pr = 0; pr < 4; ++pr) {
+                    // columns 2j and 2j+1 of this lane's packet, weight rows (2pr, 2pr+1) of the lane group
+                    lo.u[pr] = __builtin_amdgcn_perm(r.w[2 * pr + 1][j], r.w[2 * pr][j], 0x05040100u);
+                    hi.u[pr] = __builtin_amdgcn_perm(r.w[2 * pr + 1][j], r.w[2 * pr][j], 0x07060302u);
+                }
+#pragma unroll
+                for (int rb = 0; rb < kProjRB; ++rb) {
+                    union {
+                        u32x4 u;
+                        Frag f;
+                    } pa;
+                    pa.u = live ? r.x[rb] : u32x4{0u, 0u, 0u, 0u};
+                    acc[rb][2 * j] = Ops::mma(pa.f, lo.f, acc[rb][2 * j]);
+                    acc[rb][2 * j + 1] = Ops::mma(pa.f, hi.f, acc[rb][2 * j + 1]);
+                }
+            }
+        };
+        // The scheduling barriers keep the loads of the steps in step order, in the prologue as in the loop: a wait counts
+        // in issue order, and the compiler's count at the loop head is the smaller of what the two ways into it allow.
+        Step ring[kProjDepth];
+#pragma unroll
+        for (int d = 0; d < kProjDepth; ++d) {
+            issue(d, ring[d]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int st = 0; st < steps; st += kProjDepth) {
+#pragma unroll
+            for (int d = 0; d < kProjDepth; ++d) {
+                consume(ring[d], st + d < steps);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(st + d + kProjDepth, ring[d]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-    };
-    Step sa, sb;
-    issue(0, sa);
-    issue(1, sb);
-    for (int s = 0; s < steps; s += 2) {
-        consume(sa);
-        issue(s + 2, sa);
-        if (s + 1 < steps) consume(sb);
-        issue(s + 3, sb);
-    }
-    // acc[rb][e][r] is the sum of this slab for batch row (rh*2 + rb)*16 + 4 g4 + r, column 8c + e.  The slabs meet in LDS in two
-    // rounds: the upper half of the waves writes, the lower half adds its own values to the same places.
-    float* mine = part + ((ks % (kProjSlabs / 2)) * kProjRows + rh * kProjRB * 16 + 4 * g4) * kProjPitch + 8 * c;
-    if (ks >= kProjSlabs / 2) {
+        // acc[rb][e][r] is this wave's sum for batch row rb * 16 + 4 g4 + r, column 8c + e: every wave leaves its tile in LDS
+        float* mine = part + (ks * kProjRows + 4 * g4) * kProjPitch + 8 * c;
 #pragma unroll
         for (int rb = 0; rb < kProjRB; ++rb) {
 #pragma unroll
@@ -205,59 +237,29 @@ __global__ __launch_bounds__(kProjThreads) void fusedQkvHead(T* __restrict__ qOu
                 *reinterpret_cast<f32x4*>(p + 4) = f32x4{acc[rb][4][r], acc[rb][5][r], acc[rb][6][r], acc[rb][7][r]};
             }
         }
-    }
-    __syncthreads();
-    if (ks < kProjSlabs / 2) {
-#pragma unroll
-        for (int rb = 0; rb < kProjRB; ++rb) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float* p = mine + (rb * 16 + r) * kProjPitch;
-                const f32x4 u0 = *reinterpret_cast<const f32x4*>(p), u1 = *reinterpret_cast<const f32x4*>(p + 4);
-                *reinterpret_cast<f32x4*>(p) = f32x4{acc[rb][0][r], acc[rb][1][r], acc[rb][2][r], acc[rb][3][r]} + u0;
-                *reinterpret_cast<f32x4*>(p + 4) = f32x4{acc[rb][4][r], acc[rb][5][r], acc[rb][6][r], acc[rb][7][r]} + u1;
-            }
-        }
-    }
-    __syncthreads();
-
-    if (gridDim.z > 1) {
-        // this work-group only saw a part of the hidden dimension: its sums go to the workspace, the finishing kernel adds
-        // the parts
-        float* dst = hiddenPart + (static_cast<int64_t>(blockIdx.z) * a.B) * N + tile * kFD;
-        for (int idx = threadIdx.x; idx < kProjRows * kFD; idx += kProjThreads) {
-            const int r = idx / kFD, col = idx % kFD;
+        __syncthreads();
+        // the head's partial tile of this work-group: 16-byte stores, a row of the tile is 512 consecutive bytes
+        const int slot = static_cast<int>(blockIdx.x) - projFirstWg(pl, tile);
+        float* dst = hiddenPart + (static_cast<int64_t>(slot) * a.B) * N + tile * kFD;
+        for (int idx = threadIdx.x; idx < kProjRows * (kFD / 4); idx += kProjThreads) {
+            const int r = idx / (kFD / 4), col = (idx % (kFD / 4)) * 4;
             if (rowBase + r >= a.B) continue;
-            float v = 0.f;
+            f32x4 v = *reinterpret_cast<const f32x4*>(part + r * kProjPitch + col);
 #pragma unroll
-            for (int k4 = 0; k4 < kProjSlabs / 2; ++k4) v += part[(k4 * kProjRows + r) * kProjPitch + col];
-            dst[static_cast<int64_t>(rowBase + r) * N + col] = v;
+            for (int k2 = 1; k2 < kProjWaves; ++k2) v += *reinterpret_cast<const f32x4*>(part + (k2 * kProjRows + r) * kProjPitch + col);
+            *reinterpret_cast<f32x4*>(dst + static_cast<int64_t>(rowBase + r) * N + col) = v;
         }
-        return;
-    }
-    // ---- bias, rotation, and the head's destination: a thread takes the pair (j, j + 64) of a batch row
-    for (int idx = threadIdx.x; idx < kProjRows * (kFD / 2); idx += kProjThreads) {
-        const int r = idx / (kFD / 2);
-        const int j = idx % (kFD / 2);
-        const int b = rowBase + r;
-        if (b >= a.B || rowFinished(a, b)) continue;
-        float v0 = 0.f, v1 = 0.f;
-#pragma unroll
-        for (int k4 = 0; k4 < kProjSlabs / 2; ++k4) {
-            v0 += part[(k4 * kProjRows + r) * kProjPitch + j];
-            v1 += part[(k4 * kProjRows + r) * kProjPitch + j + kFD / 2];
-        }
-        finishPair<T>(qOut, kCache, vCache, bias, a, tile, b, j, v0, v1);
+        __syncthreads();  // the tile storage is free for the next head of the run
     }
 }
 
-// The second half of a projection whose hidden dimension was split over several work-groups per head: adds the parts and
-// finishes every pair as fusedQkvHead does.
+// Adds the partial tiles of a head and finishes every pair: rounding, bias, rotation, and the stores of q, k and v.
 template <typename T>
 __global__ __launch_bounds__(256) void fusedQkvFinish(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const float* __restrict__ hiddenPart,
-                                                      const T* __restrict__ bias, FusedArgs a, int parts) {
+                                                      const T* __restrict__ bias, FusedArgs a, ProjPlan pl) {
     const int tile = blockIdx.x;
-    const int N = (a.H + 2 * a.Hkv) * kFD;
+    const int N = pl.tiles * kFD;
+    const int parts = projLastWg(pl, tile) - projFirstWg(pl, tile) + 1;
     for (int idx = threadIdx.x; idx < 4 * (kFD / 2); idx += 256) {
         const int b = blockIdx.y * 4 + idx / (kFD / 2);
         const int j = idx % (kFD / 2);
@@ -352,9 +354,13 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
 #pragma unroll
         for (int r = 0; r < 8; ++r) vb[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + rowOf(kAttnStep * st + 8 * g4 + r)));
     };
+    // The scheduling barriers keep the requests in the order K, V, K, V ...: a wait for the K rows then leaves the V rows
+    // in flight and the other way round (a wait is a count of younger requests).
     if (nSteps > 0) {  // a wave without chunks (a short range) only takes part in the hand-over below
         issueK(0);
+        __builtin_amdgcn_sched_barrier(0);
         issueV(0);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     f32x4 acc[8];
@@ -385,7 +391,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
                 sc[tg] = Ops::mma(qa[s], u.f, sc[tg]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
         issueK(st + 1);  // the K registers are free: the next step's rows (past the range: its last row again)
+        __builtin_amdgcn_sched_barrier(0);
         float alpha[4];
         bool moved = false;
 #pragma unroll
@@ -432,7 +440,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
             acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
             acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
         }
+        __builtin_amdgcn_sched_barrier(0);
         issueV(st + 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- acc[e][r] is dim 8c + e of query head 4 g4 + r: the waves hand their (maximum, denominator, sums) over in LDS
@@ -510,26 +520,24 @@ __global__ __launch_bounds__(256) void fusedDecodeMerge(T* __restrict__ out, Fus
 
 template <typename T>
 diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const void* bias, void* workspace, void* kCache, void* vCache, const FusedArgs& a,
-                         const AttnSplit& spIn, int64_t qBytes, int projParts) {
+                         const AttnSplit& spIn, int64_t qBytes, const ProjPlan& pl) {
     T* qBuf = static_cast<T*>(workspace);
     AttnSplit sp = spIn;
-    // the parts of a split projection share the storage of the attention partials: the attention kernel runs after the
+    // the partial tiles of the projection share the storage of the attention partials: the attention kernel runs after the
     // finishing kernel has read them
     float* hiddenPart = reinterpret_cast<float*>(static_cast<char*>(workspace) + qBytes);
     sp.partAcc = hiddenPart;
     sp.partMl = sp.partAcc + static_cast<int64_t>(a.B) * sp.splits * a.H * kFD;
-    const size_t projLds = static_cast<size_t>(kProjSlabs / 2) * kProjRows * kProjPitch * sizeof(float);
-    ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(fusedQkvHead<T>), static_cast<int>(projLds)));
-    const dim3 pgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, kProjRows)), static_cast<unsigned>(projParts));
-    hipLaunchKernelGGL((fusedQkvHead<T>), pgrid, dim3(kProjThreads), projLds, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache), hiddenPart,
-                       static_cast<const T*>(inout), static_cast<const T*>(w), static_cast<const T*>(bias), a);
+    const size_t projLds = static_cast<size_t>(kProjWaves) * kProjRows * kProjPitch * sizeof(float);
+    ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(fusedQkvPart<T>), static_cast<int>(projLds)));
+    const int projWgs = static_cast<int>(ceilDiv(static_cast<int64_t>(pl.tiles) * pl.stepsPerTile, pl.unitsPerWg));
+    const dim3 pgrid(static_cast<unsigned>(projWgs), static_cast<unsigned>(ceilDiv(a.B, kProjRows)));
+    hipLaunchKernelGGL((fusedQkvPart<T>), pgrid, dim3(kProjThreads), projLds, stream, hiddenPart, static_cast<const T*>(inout), static_cast<const T*>(w), a, pl);
     ROCM_LAUNCH_CHECK();
-    if (projParts > 1) {
-        const dim3 fgrid(static_cast<unsigned>(a.H + 2 * a.Hkv), static_cast<unsigned>(ceilDiv(a.B, 4)));
-        hipLaunchKernelGGL((fusedQkvFinish<T>), fgrid, dim3(256), 0, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache), hiddenPart,
-                           static_cast<const T*>(bias), a, projParts);
-        ROCM_LAUNCH_CHECK();
-    }
+    const dim3 fgrid(static_cast<unsigned>(pl.tiles), static_cast<unsigned>(ceilDiv(a.B, 4)));
+    hipLaunchKernelGGL((fusedQkvFinish<T>), fgrid, dim3(256), 0, stream, qBuf, static_cast<T*>(kCache), static_cast<T*>(vCache), hiddenPart,
+                       static_cast<const T*>(bias), a, pl);
+    ROCM_LAUNCH_CHECK();
     const dim3 agrid(static_cast<unsigned>(a.Hkv), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
     hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), 0, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
                        static_cast<const T*>(vCache), a, sp);
@@ -629,16 +637,27 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     const int64_t e = vX.itemsize();
     const int64_t qBytes = ceilDiv(B * H * D * e, 256) * 256;
     const int64_t attnBytes = sp.splits > 1 ? B * sp.splits * H * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
-    // work-groups of the projection per head: the hidden dimension is cut in two as long as that does not give more
-    // work-groups than compute units (measured at 96 heads x 64 rows x 4096: 2 parts 26 us faster than 1, 4 and 8 no better;
-    // a part must still give each of a work-group's 4 slabs whole 32-row steps)
-    int projParts = 1;
-    while (projParts < 8 && (H + 2 * Hkv) * ceilDiv(B, kProjRows) * projParts * 2 <= deviceInfo().numCU && hidden % (projParts * 2 * kProjSlabs * 32) == 0 &&
-           hidden / (projParts * 2 * kProjSlabs * 32) >= 2)
-        projParts *= 2;
-    projParts = envInt("DIOPI_ROCM_FUSEDDEC_PARTS", projParts);
-    if (projParts < 1 || hidden % (projParts * kProjSlabs * 32) != 0) projParts = 1;
-    const int64_t projBytes = projParts > 1 ? projParts * B * N * static_cast<int64_t>(sizeof(float)) : 0;
+    // the projection's units in equal runs over one work-group per compute unit (fewer when a run would leave a wave without
+    // a step, or when several blocks of 64 batch rows multiply the work-groups)
+    ProjPlan pl;
+    pl.tiles = static_cast<int>(H + 2 * Hkv);
+    pl.stepsPerTile = static_cast<int>(hidden / 32);
+    {
+        const int64_t units = static_cast<int64_t>(pl.tiles) * pl.stepsPerTile;
+        const int64_t rowBlocks = ceilDiv(B > 0 ? B : 1, kProjRows);
+        // when the heads are fewer than the compute units a head is cut into as many equal runs as fit (runs that end with
+        // their head: 33.2 us at 96 heads x 4096 against 35.6 us for 256 runs that cross heads); otherwise equal runs
+        int64_t wgs = std::max<int64_t>(1, deviceInfo().numCU / rowBlocks);
+        if (pl.tiles <= wgs) wgs = pl.tiles * std::min<int64_t>(wgs / pl.tiles, ceilDiv(pl.stepsPerTile, kProjWaves));
+        wgs = envInt("DIOPI_ROCM_FUSEDDEC_WGS", static_cast<int>(wgs));
+        wgs = std::max<int64_t>(1, std::min<int64_t>(wgs, ceilDiv(units, kProjWaves)));
+        pl.unitsPerWg = static_cast<int>(ceilDiv(units, wgs));
+        if (pl.tiles <= wgs && pl.stepsPerTile % pl.unitsPerWg != 0 && pl.unitsPerWg < pl.stepsPerTile)
+            pl.unitsPerWg = static_cast<int>(ceilDiv(pl.stepsPerTile, ceilDiv(pl.stepsPerTile, pl.unitsPerWg)));  // the same count of runs per head, evened out
+        pl.slots = 1;
+        for (int t = 0; t < pl.tiles; ++t) pl.slots = std::max(pl.slots, projLastWg(pl, t) - projFirstWg(pl, t) + 1);
+    }
+    const int64_t projBytes = static_cast<int64_t>(pl.slots) * B * N * static_cast<int64_t>(sizeof(float));
     const int64_t need = qBytes + (attnBytes > projBytes ? attnBytes : projBytes);
     if (*workspace_size < 0) {
         *workspace_size = need;  // size query: nothing else happens
@@ -670,8 +689,8 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     a.layerOffset = layer_id * B * Hkv * max_seq_len * D;
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, projParts);
-    return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, projParts);
+    if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, pl);
+    return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, pl);
 }
 
 }  // namespace
