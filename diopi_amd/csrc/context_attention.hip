@@ -375,8 +375,6 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         // nothing to do for this wave: the tile lies entirely above the diagonal, or the wave's 32 rows lie past the
         // sequence (the last query tile of a sequence is rarely full; such a wave only fetches its share of the tiles)
         const bool skip = (causal && key0 > waveRowHi) || waveRowLo >= L;
-        // on its diagonal tile a wave whose rows end before the tile's second 32-key block sees only the first block
-        const bool firstBlockOnly = causal && key0 + 32 > waveRowHi;
 
         // ---- S^T = K . Q^T for the two 32-key blocks ----
         // LDS operands are requested one step ahead of the product that consumes them, and the two key blocks
@@ -402,7 +400,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
             if (st + kKDepth - 1 < kHD / 16) loadK(st + kKDepth - 1, (st + kKDepth - 1) % kKDepth);
             __builtin_amdgcn_sched_barrier(0);  // keep the read-ahead order: the scheduler would otherwise sink the reads
             s[0] = Ops::mma(kf[st % kKDepth][0].f, qf[st], s[0]);
-            if (!firstBlockOnly) s[1] = Ops::mma(kf[st % kKDepth][1].f, qf[st], s[1]);  // else masked below as a whole
+            s[1] = Ops::mma(kf[st % kKDepth][1].f, qf[st], s[1]);
             __builtin_amdgcn_sched_barrier(0);
         }
         // V^T operands of the first 16-key group travel while the softmax runs
@@ -474,7 +472,6 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int sb = g / 2, u = g % 2;
-            if (sb == 1 && firstBlockOnly) break;  // probabilities of the second block are all zero
             FragBits<Frag> pk;
             if constexpr (kFold) {
 #pragma unroll

@@ -82,6 +82,12 @@ def test_fused_decoder_attention_circular_cache_and_many_rows():
     _case(B=70, H=4, Hkv=2, S=48, seq=[(7 * i) % 200 for i in range(70)], dt=torch.float16, seed=4, step=260, what="wrap, 70 rows")
 
 
+def test_fused_decoder_attention_projection_runs_that_cross_heads():
+    # 2200 rows are 35 blocks of 64: the projection then has fewer work-groups per block (256 // 35 = 7) than heads (8), and its
+    # equal runs of (head, 32-row step) units end inside heads: a work-group writes partial tiles of two heads
+    _case(B=2200, H=4, Hkv=2, S=24, seq=[(5 * i) % 24 for i in range(2200)], dt=torch.float16, seed=9, layers=1, layer=0, what="2200 rows")
+
+
 def test_fused_decoder_attention_decode_shape_sampled():
     """The decode benchmark's shape (batch 64, 32 heads of 128, hidden 4096, lengths 512..2047 in a 2048-row cache): the whole
     output against the oracle."""
