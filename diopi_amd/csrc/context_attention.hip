@@ -134,6 +134,15 @@ __device__ __forceinline__ float maxWithOtherHalf(float v) {
     return fmaxf(lo, hi);
 }
 
+// max(a, b, c) as the one instruction it is.  Written out because fmaxf on values the compiler cannot prove to be
+// quiet numbers first canonicalises each of them (a v_max_f32 x, x, x apiece: 12 extra vector instructions per key tile);
+// the scores are sums of finite products or the mask's -1e30, never signalling NaNs.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // Sequence geometry with every value forced inside the tensors.
 struct SeqInfo {
     int64_t start;
@@ -437,11 +446,16 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
         float tm[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            tm[c] = fmaxf(s[c / 2][8 * (c % 2)], s[c / 2][8 * (c % 2) + 1]);
-#pragma unroll
-            for (int r = 2; r < 8; ++r) tm[c] = fmaxf(tm[c], s[c / 2][8 * (c % 2) + r]);
+            const int sb = c / 2, r0 = 8 * (c % 2);
+            tm[c] = max3(s[sb][r0], s[sb][r0 + 1], s[sb][r0 + 2]);
+            tm[c] = max3(tm[c], s[sb][r0 + 3], s[sb][r0 + 4]);
+            tm[c] = max3(tm[c], s[sb][r0 + 5], s[sb][r0 + 6]);
         }
-        const float tmax = maxWithOtherHalf(fmaxf(fmaxf(tm[0], tm[1]), fmaxf(tm[2], tm[3])));
+        const float tmA = max3(tm[0], s[0][7], s[0][15]), tmB = max3(tm[1], s[1][7], s[1][15]);
+        float tmLo = max3(max3(tmA, tmB, tm[2]), tm[3], tm[3]);  // this lane's 32 scores
+        float tmHi = tmLo;
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(tmLo), "+v"(tmHi));  // see maxWithOtherHalf
+        const float tmax = max3(tmLo, tmHi, tmHi);
         // The reference only follows the true maximum when it has fallen behind by more than 2^kLazyLog2 (a
         // wave-uniform, rarely taken branch after the first tile, where it is set for the first time): probabilities
         // then reach at most 2^kLazyLog2, which the 16-bit types hold with full relative precision, and the
