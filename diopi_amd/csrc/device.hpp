@@ -152,6 +152,53 @@ __device__ __forceinline__ int64_t loadIndex(const void* base, int64_t i, bool i
     return is64 ? reinterpret_cast<const int64_t*>(base)[i] : static_cast<int64_t>(reinterpret_cast<const int32_t*>(base)[i]);
 }
 
+// Longest first.  Work-groups start in the order of their index and a compute unit holds a few at a time, so when their
+// work is ragged the order decides how long the last ones run alone.  Called by all 64 lanes of one wave: returns which
+// of n <= 256 items (4 per lane) has the r-th largest size, ties by item number, by bisection on the size (sizeOf(j) in
+// [0, maxSize]): log2(maxSize) rounds of 4 compares and 4 ballots, a few hundred instructions that the streaming of the
+// other resident work-groups hides.  Every r in [0, n) gets a different item.
+constexpr int kRankedItems = 4 * kWave;
+template <typename SizeOf>
+__device__ __forceinline__ int itemOfRank(int r, int n, int maxSize, SizeOf sizeOf) {
+    const int l = threadIdx.x % kWave;
+    int sz[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int j = l + kWave * k;
+        sz[k] = j < n ? sizeOf(j) : -1;  // no such item: behind every real one
+    }
+    auto atLeast = [&](int v) {  // items of at least this size
+        int c = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) c += __builtin_popcountll(__ballot(sz[k] >= v));
+        return c;
+    };
+    int lo = 0, hi = maxSize + 1;  // atLeast(lo) > r >= atLeast(hi)
+    while (hi - lo > 1) {
+        const int mid = lo + (hi - lo) / 2;
+        if (atLeast(mid) > r) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    int t = r - atLeast(lo + 1);  // position among the items of exactly this size
+    int found = r;
+    bool done = false;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const unsigned long long eq = __ballot(sz[k] == lo);
+        const int before = __builtin_popcountll(eq & ((1ull << l) - 1ull));
+        const unsigned long long hit = __ballot(sz[k] == lo && before == t);
+        if (!done && hit != 0ull) {
+            found = __builtin_ctzll(hit) + kWave * k;
+            done = true;
+        }
+        t -= __builtin_popcountll(eq);
+    }
+    return found;
+}
+
 // The same without a branch: two loads whatever the width (for 32-bit storage the second one re-reads the element),
 // combined afterwards.  A load inside a branch makes the compiler wait for it before the branch ends; this form lets
 // the value stay in flight until its first use.

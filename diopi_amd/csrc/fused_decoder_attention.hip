@@ -27,7 +27,7 @@
 //                    in LDS (fp32, 132 KiB) and the work-group writes one fp32 partial tile per head its run touched.
 //   fusedQkvFinish   adds the partial tiles of a head, rounds, adds the bias, rotates, and writes the head: q to the
 //                    workspace, k and v straight into the cache.
-//   fusedDecodeAttn  a work-group owns (batch row, kv head, range of 512 cached tokens) and its four waves take the range's
+//   fusedDecodeAttn  a work-group owns (batch row, kv head, range of 1024 cached tokens; the items longest first) and its four waves take the range's
 //                    128-token chunks in turn, meeting only for a final hand-over in LDS; per 32 tokens 8 K loads that arrive in
 //                    the B-operand layout of q.k^T (16 lanes x 16-byte pieces of 16 consecutive cache rows), online
 //                    softmax on the 16 x 32 scores (row maxima and sums by DPP row reductions), probabilities through a
@@ -289,11 +289,35 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
     using Frag = typename Ops::Frag;
     __shared__ __attribute__((aligned(16))) T sP[kAttnWaves][16 * kProbPitch];
     __shared__ __attribute__((aligned(16))) float sMerge[kAttnWaves][16][kFD + 4];  // per wave and query head: 128 sums, maximum, denominator
-    const int b = blockIdx.y;
-    const int split = blockIdx.z;
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int hk = blockIdx.x;  // the kv head of this work-group
+    // the (row, range) of this work-group: longest first when the items can be ranked (see itemOfRank), else as they come
+    __shared__ int sItem;
+    int item = static_cast<int>(blockIdx.z) * a.B + static_cast<int>(blockIdx.y);
+    if (a.B * sp.splits > 1 && a.B <= kRankedItems) {
+        if (wave == 0) {
+            auto windowOf = [&](int row) {
+                if (rowFinished(a, row)) return 0;
+                const int64_t len = rowLength(a, row);
+                return static_cast<int>(len + 1 < a.maxSeq ? len + 1 : a.maxSeq);
+            };
+            int picked;
+            if (a.B * sp.splits <= kRankedItems) {
+                picked = itemOfRank(item, a.B * sp.splits, sp.TT, [&](int j) {
+                    const int rest = windowOf(j % a.B) - (j / a.B) * sp.TT;
+                    return rest <= 0 ? 0 : (rest < sp.TT ? rest : sp.TT);
+                });
+            } else {
+                picked = static_cast<int>(blockIdx.z) * a.B + itemOfRank(static_cast<int>(blockIdx.y), a.B, a.maxSeq, windowOf);
+            }
+            if (threadIdx.x == 0) sItem = picked;
+        }
+        __syncthreads();
+        item = sItem;
+    }
+    const int b = item % a.B;
+    const int split = item / a.B;
     if (rowFinished(a, b)) return;
     const int64_t L = rowLength(a, b);
     const int nWin = static_cast<int>(L + 1 < a.maxSeq ? L + 1 : a.maxSeq);  // tokens in the window, the new one last
@@ -623,11 +647,11 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
                      static_cast<long long>(hidden));
         return diopiNoImplement;
     }
-    // ranges of the attention kernel: 512 cached tokens per work-group (its four waves share them), the workspace sized for
-    // max_seq_len.  Measured at 64 rows of 511..2047 tokens, 32 kv heads: 256..1024 tokens per range within 1.5 us of each
-    // other, 2048 (no partials, no merge launch) 7 us slower: rows of unequal length then leave the last work-groups alone
+    // ranges of the attention kernel: 1024 cached tokens per work-group (its four waves share them), the workspace sized for
+    // max_seq_len.  Measured at 64 rows of 512..2047 tokens, 32 kv heads, items taken longest first: 1024 tokens per range
+    // 237-238 us per call in two harnesses, 512: 247-251, 2048 (no partials, no merge launch): 235 in one, 254 in the other
     AttnSplit sp;
-    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 512);
+    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 1024);
     sp.TT = static_cast<int>(ceilDiv(sp.TT, kAttnStep)) * kAttnStep;
     sp.splits = static_cast<int>(ceilDiv(max_seq_len, sp.TT));
     sp.partAcc = nullptr;

@@ -88,16 +88,45 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     __shared__ __attribute__((aligned(16))) float sMerge[kRvWaves][GC][kMergePitch];  // per wave and query head: 128 sums, maximum, denominator
 
     // x runs over kv heads (neighbouring work-groups read neighbouring 256-byte pieces of the same cache rows at the same
-    // time), y over sequences, z over token ranges, with the sequence rotated by the range index so that consecutive
-    // work-groups (dealt round-robin to the 8 XCDs) mix ranges of different sequences: with ragged lengths no XCD is
-    // left with only the sparse late ranges
-    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    // time), y and z over the (sequence, range) items
+    const int waveId = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    // Which (sequence, range) is this work-group's?  The one whose token count has the rank of the work-group's index
+    // (y, then z: the order in which work-groups start), over all items when there are at most 256, else over the
+    // sequences of each range (a range's token counts fall with the sequence length like the lengths themselves);
+    // with more sequences than that the items are taken as they come, the sequence rotated by the range so that
+    // neighbouring work-groups mix ranges of different sequences.
+    __shared__ int sItem;
+    const int nSeq = static_cast<int>(gridDim.y);
+    const int nItems = nSeq * static_cast<int>(gridDim.z);
+    int item = static_cast<int>(blockIdx.z) * nSeq + static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    if (nItems > 1 && nSeq <= kRankedItems) {
+        if (waveId == 0) {
+            auto lengthOf = [&](int seq) {
+                const int64_t len = loadIndex(a.bSeqLen, seq, a.len64);
+                return len > a.maxInputLen ? a.maxInputLen : (len < 0 ? int64_t{0} : len);
+            };
+            int picked;
+            if (nItems <= kRankedItems) {
+                picked = itemOfRank(static_cast<int>(blockIdx.z) * nSeq + static_cast<int>(blockIdx.y), nItems, sp.TT, [&](int j) {
+                    const int64_t rest = lengthOf(j % nSeq) - static_cast<int64_t>(j / nSeq) * sp.TT;
+                    return rest <= 0 ? 0 : (rest < sp.TT ? static_cast<int>(rest) : sp.TT);
+                });
+            } else {
+                picked = static_cast<int>(blockIdx.z) * nSeq +
+                         itemOfRank(static_cast<int>(blockIdx.y), nSeq, static_cast<int>(a.maxInputLen), [&](int j) { return static_cast<int>(lengthOf(j)); });
+            }
+            if (threadIdx.x == 0) sItem = picked;
+        }
+        __syncthreads();
+        item = sItem;
+    }
+    const int i = item % nSeq;
+    const int zIdx = item / nSeq;
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * sp.TT;
+    const int64_t t0 = static_cast<int64_t>(zIdx) * sp.TT;
     const int HG = sp.headsPerGroup;
     const int phases = kRvWaves / HG;  // waves that share a kv head take the sub-tiles in turn
-    const int waveId = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int hkRaw = blockIdx.x * HG + waveId % HG;
     const bool headLive = hkRaw < a.Hkv;
     const int hk = headLive ? hkRaw : a.Hkv - 1;  // a wave past the last kv head streams nothing and writes nothing
@@ -105,7 +134,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     if (t0 >= L) {
         // a sequence without tokens: the reference's product over an empty inner dimension gives zeros
         // (functions_lightllm.cpp:98-104); the work-groups of range 0 write them
-        if (L <= 0 && blockIdx.z == 0 && phase == 0 && headLive) {
+        if (L <= 0 && zIdx == 0 && phase == 0 && headLive) {
             const int l = threadIdx.x % kWave;
             Pack16<T> z;
             z.raw = u32x4{0u, 0u, 0u, 0u};
@@ -354,7 +383,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         if (single) {
             out[(static_cast<int64_t>(i) * a.H + qh) * kD + d] = static_cast<T>(num / den);
         } else {
-            const int64_t slot = (static_cast<int64_t>(i) * sp.splits + blockIdx.z) * a.H + qh;
+            const int64_t slot = (static_cast<int64_t>(i) * sp.splits + zIdx) * a.H + qh;
             sp.partAcc[slot * kD + d] = num;
             if (d == 0) {
                 sp.partMl[slot * 2] = m;
