@@ -55,6 +55,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-diagnostic", action="store_true", help="skip the entries marked diagnostic (counter runs: they launch the same kernels on other data)")
     ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,penalty,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
@@ -524,18 +525,20 @@ def main():
         record("diopiContextAttentionInference", f"cfg4 tokens in bf16 B=8 T={w4['T']}", ms_b, flops, "mfma", "bf16", None)
         # diagnostic, not a result: the fp16 kernel once more on all-zero tensors of the same shape.  The instruction stream is
         # the same; what differs is the data-dependent switching in the matrix pipes, and with it the clock the power limit allows
-        qz, kz, vz = (torch.zeros_like(w4[k]) for k in ("q", "k", "v"))
-        hz = {k: Tensor(v) for k, v in dict(q=qz, k=kz, v=vz).items()}
+        if not args.no_diagnostic:
+            qz, kz, vz = (torch.zeros_like(w4[k]) for k in ("q", "k", "v"))
+            hz = {k: Tensor(v) for k, v in dict(q=qz, k=kz, v=vz).items()}
 
-        def pre_zero(i):
-            check(impl.diopiContextAttentionInference(ctx.handle, h["out"].handle, hz["q"].handle, hz["k"].handle, hz["v"].handle, h["b_start_loc"].handle,
-                                                      h["b_seq_len"].handle, w4["max_input_len"]), "diopiContextAttentionInference")
-            ctx.clear_tensors()
+            def pre_zero(i):
+                check(impl.diopiContextAttentionInference(ctx.handle, h["out"].handle, hz["q"].handle, hz["k"].handle, hz["v"].handle,
+                                                          h["b_start_loc"].handle, h["b_seq_len"].handle, w4["max_input_len"]), "diopiContextAttentionInference")
+                ctx.clear_tensors()
 
-        ms_z = timed(pre_zero)
-        record("diopiContextAttentionInference", f"cfg4 shape, all-zero q/k/v (diagnostic) B=8 T={w4['T']}", ms_z, flops, "mfma", "f16", None,
-               note="not a result: same instruction stream as the cfg4 entry without data-dependent switching; the gap to the cfg4 entry is clock")
-        del w4, hf, k8, v8, lse, hb, qb, kb, vb, ob, hz, qz, kz, vz
+            ms_z = timed(pre_zero)
+            record("diopiContextAttentionInference", f"cfg4 shape, all-zero q/k/v (diagnostic) B=8 T={w4['T']}", ms_z, flops, "mfma", "f16", None,
+                   note="not a result: same instruction stream as the cfg4 entry without data-dependent switching; the gap to the cfg4 entry is clock")
+            del hz, qz, kz, vz
+        del w4, hf, k8, v8, lse, hb, qb, kb, vb, ob
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ the JSON line
