@@ -646,6 +646,32 @@ def test_decode_config3_scaled_and_ragged():
     _decode_case(w2, torch.float16, "ragged lengths")
 
 
+def test_decode_work_order_with_many_sequences_and_many_ranges():
+    """The second decode operator hands its (sequence, range) items to the work-groups longest first when it can rank them:
+    all items up to 256, the sequences of each range up to 256 sequences, nothing beyond.  Each of the three ways must give
+    every item to exactly one work-group: the whole output against the oracle, with ties among the lengths and empty
+    sequences in every case."""
+    rng = np.random.Generator(np.random.PCG64(91))
+
+    def case(B, lo, hi, what, fixed=()):
+        lens = rng.integers(lo, hi + 1, size=B).astype(np.int32)
+        for pos, val in fixed:
+            lens[pos] = val
+        w = W._decode(DEV, 90 + B, torch.float16, B, 2, 2, 128, B * hi, 1, hi, B)
+        w["b_seq_len"] = torch.from_numpy(lens).to(DEV)
+        w["b_start_loc"] = torch.from_numpy(np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int32)).to(DEV)
+        w["total_len"] = int(lens.sum())
+        w["max_input_len"] = int(hi)
+        _decode_case(w, torch.float16, what)
+
+    # 3 ranges of 2048 tokens x 100 sequences = 300 items: ranked per range
+    case(100, 1, 5000, "100 sequences x 3 ranges", fixed=((0, 0), (1, 2048), (2, 2048), (3, 2049), (4, 4096), (5, 5000), (6, 5000), (99, 0)))
+    # 300 sequences of one range: taken as they come
+    case(300, 1, 200, "300 short sequences", fixed=((0, 0), (7, 200), (8, 200), (299, 0)))
+    # 2 ranges x 128 sequences = 256 items: all ranked together, many ties
+    case(128, 2040, 2056, "128 sequences x 2 ranges, lengths within 16 of each other", fixed=((5, 0), (6, 1)))
+
+
 def test_decode_gqa_config5_scaled():
     w = W.cfg5(DEV, seed=5, scale=1 / 32)  # 4 sequences of 1024..8192 tokens, 64 q heads over 8 kv heads
     _decode_case(w, torch.bfloat16, "cfg5 x 1/32")
