@@ -294,8 +294,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
     const int hk = blockIdx.x;  // the kv head of this work-group
     // the (row, range) of this work-group: longest first when the items can be ranked (see itemOfRank), else as they come
     __shared__ int sItem;
-    int item = static_cast<int>(blockIdx.z) * a.B + static_cast<int>(blockIdx.y);
-    if (a.B * sp.splits > 1 && a.B <= kRankedItems) {
+    int b = static_cast<int>(blockIdx.y), split = static_cast<int>(blockIdx.z);
+    if (a.B <= kRankedItems && a.B * sp.splits > 1) {  // at most 256 x 65535 items: no overflow
         if (wave == 0) {
             auto windowOf = [&](int row) {
                 if (rowFinished(a, row)) return 0;
@@ -304,20 +304,19 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
             };
             int picked;
             if (a.B * sp.splits <= kRankedItems) {
-                picked = itemOfRank(item, a.B * sp.splits, sp.TT, [&](int j) {
+                picked = itemOfRank(split * a.B + b, a.B * sp.splits, sp.TT, [&](int j) {
                     const int rest = windowOf(j % a.B) - (j / a.B) * sp.TT;
                     return rest <= 0 ? 0 : (rest < sp.TT ? rest : sp.TT);
                 });
             } else {
-                picked = static_cast<int>(blockIdx.z) * a.B + itemOfRank(static_cast<int>(blockIdx.y), a.B, a.maxSeq, windowOf);
+                picked = split * a.B + itemOfRank(b, a.B, a.maxSeq, windowOf);
             }
             if (threadIdx.x == 0) sItem = picked;
         }
         __syncthreads();
-        item = sItem;
+        b = sItem % a.B;
+        split = sItem / a.B;
     }
-    const int b = item % a.B;
-    const int split = item / a.B;
     if (rowFinished(a, b)) return;
     const int64_t L = rowLength(a, b);
     const int nWin = static_cast<int>(L + 1 < a.maxSeq ? L + 1 : a.maxSeq);  // tokens in the window, the new one last
@@ -579,7 +578,7 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
                                    diopiTensorHandle_t value_cache, diopiConstTensorHandle_t finished, diopiConstTensorHandle_t total_padding_tokens,
                                    diopiConstTensorHandle_t sequence_lengths, int64_t step, int64_t layer_id, int64_t local_head_num,
                                    int64_t local_kv_head_num, int64_t size_per_head, int64_t max_seq_len, int64_t rotary_embedding, float rope_theta) {
-    (void)fusion_level;  // every level gets the same three kernels
+    (void)fusion_level;  // every level gets the same kernels
     TensorView vX, vW, vB, vWs, vK, vV, vF, vP, vL;
     ROCM_CALL(unwrap(inoutput, "inoutput", &vX));
     ROCM_CALL(unwrap(qkv_weight, "qkv_weight", &vW));
@@ -635,7 +634,7 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
         a.pad64 = vP.dtype == diopi_dtype_int64;
     }
     // what this build implements: 16-bit elements, heads of 128, up to 16 query heads per kv head, rotation of the whole head
-    // or none, a hidden size that the projection's 4 slabs of 32-row steps divide, 16-byte aligned rows
+    // or none, a hidden size in whole 32-row steps for each of a work-group's four waves, 16-byte aligned rows
     const bool supported = (vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16) && D == kFD && H / Hkv <= 16 &&
                            (rotary_embedding == 0 || rotary_embedding == kFD) && hidden % 128 == 0 && hidden >= 256 &&
                            ((reinterpret_cast<uintptr_t>(vX.data) | reinterpret_cast<uintptr_t>(vW.data) | reinterpret_cast<uintptr_t>(vK.data) |

@@ -97,17 +97,18 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     // neighbouring work-groups mix ranges of different sequences.
     __shared__ int sItem;
     const int nSeq = static_cast<int>(gridDim.y);
-    const int nItems = nSeq * static_cast<int>(gridDim.z);
-    int item = static_cast<int>(blockIdx.z) * nSeq + static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
-    if (nItems > 1 && nSeq <= kRankedItems) {
+    const int nRanges = static_cast<int>(gridDim.z);
+    int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    int zIdx = static_cast<int>(blockIdx.z);
+    if (nSeq <= kRankedItems && nSeq * nRanges > 1) {  // at most 256 x 65535 items: no overflow
         if (waveId == 0) {
             auto lengthOf = [&](int seq) {
                 const int64_t len = loadIndex(a.bSeqLen, seq, a.len64);
                 return len > a.maxInputLen ? a.maxInputLen : (len < 0 ? int64_t{0} : len);
             };
             int picked;
-            if (nItems <= kRankedItems) {
-                picked = itemOfRank(static_cast<int>(blockIdx.z) * nSeq + static_cast<int>(blockIdx.y), nItems, sp.TT, [&](int j) {
+            if (nSeq * nRanges <= kRankedItems) {
+                picked = itemOfRank(static_cast<int>(blockIdx.z) * nSeq + static_cast<int>(blockIdx.y), nSeq * nRanges, sp.TT, [&](int j) {
                     const int64_t rest = lengthOf(j % nSeq) - static_cast<int64_t>(j / nSeq) * sp.TT;
                     return rest <= 0 ? 0 : (rest < sp.TT ? static_cast<int>(rest) : sp.TT);
                 });
@@ -118,10 +119,9 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
             if (threadIdx.x == 0) sItem = picked;
         }
         __syncthreads();
-        item = sItem;
+        i = sItem % nSeq;
+        zIdx = sItem / nSeq;
     }
-    const int i = item % nSeq;
-    const int zIdx = item / nSeq;
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
     const int64_t t0 = static_cast<int64_t>(zIdx) * sp.TT;
