@@ -21,7 +21,7 @@ def say(*a):
 
 
 def _case(B, H, Hkv, S, seq, dt, seed, hidden=None, layers=2, layer=1, pad=None, finished=None, step=None, bias=True, rot=128, idt=torch.int32,
-          theta=10000.0, what=""):
+          theta=10000.0, what="", out_mismatch=0.0):
     D = 128
     g = torch.Generator().manual_seed(seed)
     hid = H * D if hidden is None else hidden
@@ -48,8 +48,8 @@ def _case(B, H, Hkv, S, seq, dt, seed, hidden=None, layers=2, layer=1, pad=None,
     out = F.fused_decoder_attention_inp(xd, wd, bd, None, 0, kd, vd, args[0], args[1], args[2], step, layer, H, Hkv, D, S, rot, theta)
     assert_bit_equal(wd, w_before, "qkv_weight was modified")
     tol = TOL[dt]
-    assert_close(out, ref, what=what + " output vs reference composition", **tol)
-    assert_close(out, ex, what=what + " output vs float64", **tol)
+    assert_close(out, ref, what=what + " output vs reference composition", mismatch_ratio=out_mismatch, **tol)
+    assert_close(out, ex, what=what + " output vs float64", mismatch_ratio=out_mismatch, **tol)
     say(what, "max_abs/rel vs f64: %.3e %.3e" % report(out, ex))
     # caches: the written rows within tolerance, every other row untouched
     written = torch.zeros(layers, B, Hkv, S, dtype=torch.bool)
@@ -86,6 +86,35 @@ def test_fused_decoder_attention_projection_runs_that_cross_heads():
     # 2200 rows are 35 blocks of 64: the projection then has fewer work-groups per block (256 // 35 = 7) than heads (8), and its
     # equal runs of (head, 32-row step) units end inside heads: a work-group writes partial tiles of two heads
     _case(B=2200, H=4, Hkv=2, S=24, seq=[(5 * i) % 24 for i in range(2200)], dt=torch.float16, seed=9, layers=1, layer=0, what="2200 rows")
+
+
+def test_fused_decoder_attention_random_shapes():
+    """Twelve seeded random combinations of batch, head grouping, cache length, hidden size, lengths (before and past the wrap),
+    finished rows, padding offsets, rotation on or off, bias or none, index width and dtype.  With bf16 tensors 2 in 1000
+    output elements may miss the bar: over a window of a handful of tokens nothing averages out, and one bf16 rounding of a score
+    of size 4 (the composition keeps its scores in the tensor type; the device rounds q and k to it) moves a probability by 2 %."""
+    rng = torch.Generator().manual_seed(1234)
+
+    def pick(*vals):
+        return vals[int(torch.randint(len(vals), (1,), generator=rng))]
+
+    for n in range(12):
+        Hkv = pick(1, 2, 3, 4)
+        G = pick(1, 2, 4, 5, 8, 16)
+        H = Hkv * G
+        B = pick(1, 2, 7, 33, 65)
+        S = pick(16, 31, 100, 257, 600, 1100)
+        extra = pick(0, 0, 128, 384)
+        hidden = max(H * 128 + extra, 256)
+        wrap = pick(False, False, True)
+        hi = 3 * S if wrap else S - 1
+        seq = torch.randint(0, hi + 1, (B,), generator=rng).tolist()
+        finished = None if pick(True, False) else (torch.rand(B, generator=rng) < 0.3).tolist()
+        pad = None if pick(True, False) else torch.randint(0, 5, (B,), generator=rng).tolist()
+        dt = pick(torch.float16, torch.bfloat16)
+        _case(B=B, H=H, Hkv=Hkv, S=S, seq=seq, dt=dt, seed=100 + n, hidden=hidden, layers=pick(1, 3), layer=0,
+              pad=pad, finished=finished, step=max(seq) + 1 + (0 if pad is None else 5), bias=pick(True, False), rot=pick(0, 128),
+              idt=pick(torch.int32, torch.int64), what=f"random case {n}", out_mismatch=2e-3 if dt is torch.bfloat16 else 0.0)
 
 
 def test_fused_decoder_attention_decode_shape_sampled():
