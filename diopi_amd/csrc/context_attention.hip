@@ -47,7 +47,6 @@ constexpr int kBN = 64;    // key rows per tile
 constexpr int kHD = 128;   // head size of the MFMA kernel
 constexpr int kLD = kHD + 8;  // row pitch of the output tile in LDS, in elements (272 bytes: 16-byte aligned)
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-constexpr int kNumXcd = 8;
 constexpr float kLazyLog2 = 8.0f;  // how far (in powers of two) the softmax reference maximum may lag behind
 
 struct CtxArgs {

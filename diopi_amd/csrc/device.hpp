@@ -10,6 +10,7 @@
 namespace rocm {
 
 constexpr int kWave = 64;  // CDNA wavefront width
+constexpr int kNumXcd = 8;  // accelerator dies of an MI355X: consecutive work-groups of a launch go to them round-robin
 
 using half_t = _Float16;
 using bf16_t = __bf16;

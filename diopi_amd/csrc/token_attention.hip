@@ -182,7 +182,7 @@ constexpr int kStagePitch = 136;  // elements per staged row: 128 + 8
 
 template <typename T, int HW>
 __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, DecodeArgs a, int TT,
-                                                              int HS, float scale) {
+                                                              int HS, float scale, int order) {
     using Ops = MfmaOps<T>;
     using Frag = typename Ops::Frag;
     constexpr int D = 128;
@@ -195,13 +195,21 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     extern __shared__ __attribute__((aligned(16))) unsigned char dynLds[];  // scores of the tile: HS*HW*G rows of TT + 8
 
     // x runs over head groups (neighbouring work-groups read neighbouring pieces of the same cache rows at the same
-    // time), y over sequences, z over token tiles, with the sequence rotated by the tile index so that consecutive
-    // work-groups (which the dispatcher deals round-robin to the 8 XCDs) mix tiles of different sequences: with
-    // ragged lengths no XCD is left with only the sparsely populated late tiles
-    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    // time); the launcher says how y and z map to (sequence, token tile)
+    int i, tileIdx;
+    if (order == 1) {  // y = tile, z = sequence: the tiles of a sequence one after the other
+        i = static_cast<int>(blockIdx.z);
+        tileIdx = static_cast<int>(blockIdx.y);
+    } else if (order == 3) {  // y = sequence, z = tile
+        i = static_cast<int>(blockIdx.y);
+        tileIdx = static_cast<int>(blockIdx.z);
+    } else {  // y = sequence, z = tile, the sequence rotated by the tile index: consecutive work-groups mix tiles of different sequences
+        i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+        tileIdx = static_cast<int>(blockIdx.z);
+    }
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
-    const int64_t t0 = static_cast<int64_t>(blockIdx.z) * TT;
+    const int64_t t0 = static_cast<int64_t>(tileIdx) * TT;
     if (t0 >= L) return;
     const int nTok = static_cast<int>((L - t0 < TT) ? L - t0 : TT);
     const int64_t start = loadIndex(a.bStartLoc, i, a.start64);
@@ -409,10 +417,18 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     while (TT > 64 && outRows * (TT + 8) * static_cast<int>(sizeof(T)) > 40 * 1024) TT -= 64;
     const size_t outLds = static_cast<size_t>(outRows) * (TT + 8) * sizeof(T);
     ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
-    const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
+    // Work-groups go round-robin to the 8 XCDs in index order.  When the head groups (x) are a multiple of 8, a work-group's XCD
+    // depends on its head group alone and every XCD gets the same share whatever the order of the rest: the tiles of a
+    // sequence then run one after the other, y = tile, z = sequence (cfg3: 100.3 us against 103.1).  Otherwise a
+    // sequence would stay on a few XCDs and ragged lengths would unbalance them: y = sequence, z = tile, the sequence rotated by
+    // the tile index (cfg5, 2 head groups: 242 us; unrotated 264, tiles in sequence order 268).
+    const int gridX = static_cast<int>(ceilDiv(a.Hkv, HS * HW));
+    const int order = envInt("DIOPI_ROCM_TOKATT_ORDER", gridX % kNumXcd == 0 ? 1 : 0);
+    const dim3 grid = order == 1 ? dim3(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch))
+                                 : dim3(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
 #define ROCM_STAGED_CASE(HWC)                                                                                                                         \
     hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), outLds, stream, static_cast<T*>(out), static_cast<const T*>(q),             \
-                       static_cast<const T*>(k), a, TT, HS, scale)
+                       static_cast<const T*>(k), a, TT, HS, scale, order)
     if (HW == 4) {
         ROCM_STAGED_CASE(4);
     } else if (HW == 2) {
