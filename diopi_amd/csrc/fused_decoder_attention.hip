@@ -288,7 +288,9 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
     using Ops = Mfma16<T>;
     using Frag = typename Ops::Frag;
     __shared__ __attribute__((aligned(16))) T sP[kAttnWaves][16 * kProbPitch];
-    __shared__ __attribute__((aligned(16))) float sMerge[kAttnWaves][16][kFD + 4];  // per wave and query head: 128 sums, maximum, denominator
+    // per wave and query head of the group: 128 sums, maximum, denominator; [kAttnWaves][G][kFD + 4] floats, sized by the launcher
+    // (a fixed 16 heads would cost a group of one three quarters of the work-groups a compute unit can hold)
+    extern __shared__ __attribute__((aligned(16))) float sMerge[];
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int hk = blockIdx.x;  // the kv head of this work-group
@@ -470,7 +472,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
 
     // ---- acc[e][r] is dim 8c + e of query head 4 g4 + r: the waves hand their (maximum, denominator, sums) over in LDS
     {
-        float* mine = &sMerge[wave][0][0];
+        float* mine = sMerge + wave * a.G * (kFD + 4);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int g = 4 * g4 + r;
@@ -492,15 +494,15 @@ __global__ __launch_bounds__(kAttnThreads, 2) void fusedDecodeAttn(T* __restrict
         float m = -INFINITY;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
-            mw[w] = sMerge[w][g][kFD];
+            mw[w] = sMerge[(w * a.G + g) * (kFD + 4) + kFD];
             m = fmaxf(m, mw[w]);
         }
         float num = 0.f, den = 0.f;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
             const float wgt = (mw[w] == -INFINITY) ? 0.f : __expf(mw[w] - m);  // a wave without tokens weighs nothing
-            num += wgt * sMerge[w][g][d];
-            den += wgt * sMerge[w][g][kFD + 1];
+            num += wgt * sMerge[(w * a.G + g) * (kFD + 4) + d];
+            den += wgt * sMerge[(w * a.G + g) * (kFD + 4) + kFD + 1];
         }
         const int qh = hk * G + g;
         if (single) {
@@ -562,7 +564,8 @@ diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const v
                        static_cast<const T*>(bias), a, pl);
     ROCM_LAUNCH_CHECK();
     const dim3 agrid(static_cast<unsigned>(a.Hkv), static_cast<unsigned>(a.B), static_cast<unsigned>(sp.splits));
-    hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), 0, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
+    const size_t mergeLds = static_cast<size_t>(kAttnWaves) * a.G * (kFD + 4) * sizeof(float);
+    hipLaunchKernelGGL((fusedDecodeAttn<T>), agrid, dim3(kAttnThreads), mergeLds, stream, static_cast<T*>(inout), qBuf, static_cast<const T*>(kCache),
                        static_cast<const T*>(vCache), a, sp);
     ROCM_LAUNCH_CHECK();
     if (sp.splits > 1) {
