@@ -168,15 +168,15 @@ __device__ __forceinline__ int itemOfRank(int r, int n, int maxSize, SizeOf size
         const int j = l + kWave * k;
         sz[k] = j < n ? sizeOf(j) : -1;  // no such item: behind every real one
     }
-    auto atLeast = [&](int v) {  // items of at least this size
+    auto atLeast = [&](int64_t v) {  // items of at least this size
         int c = 0;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) c += __builtin_popcountll(__ballot(sz[k] >= v));
+        for (int k = 0; k < 4; ++k) c += __builtin_popcountll(__ballot(static_cast<int64_t>(sz[k]) >= v));
         return c;
     };
-    int lo = 0, hi = maxSize + 1;  // atLeast(lo) > r >= atLeast(hi)
+    int64_t lo = 0, hi = static_cast<int64_t>(maxSize) + 1;  // atLeast(lo) > r >= atLeast(hi); 64 bits: maxSize may be INT32_MAX
     while (hi - lo > 1) {
-        const int mid = lo + (hi - lo) / 2;
+        const int64_t mid = lo + (hi - lo) / 2;
         if (atLeast(mid) > r) {
             lo = mid;
         } else {
@@ -188,9 +188,9 @@ __device__ __forceinline__ int itemOfRank(int r, int n, int maxSize, SizeOf size
     bool done = false;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const unsigned long long eq = __ballot(sz[k] == lo);
+        const unsigned long long eq = __ballot(static_cast<int64_t>(sz[k]) == lo);
         const int before = __builtin_popcountll(eq & ((1ull << l) - 1ull));
-        const unsigned long long hit = __ballot(sz[k] == lo && before == t);
+        const unsigned long long hit = __ballot(static_cast<int64_t>(sz[k]) == lo && before == t);
         if (!done && hit != 0ull) {
             found = __builtin_ctzll(hit) + kWave * k;
             done = true;

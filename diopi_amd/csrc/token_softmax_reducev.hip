@@ -507,8 +507,8 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     // writes are dear next to the row gather (8.5 MB of them cost 10 us of 111 at 64 sequences of 512..2048 tokens and
     // one query head per kv head; 19 MB cost 27 us of 236 at 128 sequences of 1024..8192 tokens and 8 query heads per
     // kv head): ranges are long, and the four waves of a work-group share one so that it still streams quickly.
-    // Measured: ranges of 2560..5120 tokens 227-229 us at the second shape (6144: 231, 8192: 243 - too few work-groups),
-    // 768..4096 tokens 107.5-110 us at the first.
+    // Measured with the items taken longest first: ranges of 4096..6144 tokens 212-215 us at the second shape (8192: 218; 2048
+    // and 3072, whose items are too many to be ranked together: 233 and 228), 2048 tokens 106 us at the first (1024: 111).
     int TT = 512 * a.G;
     if (TT < 2048) TT = 2048;
     if (TT > 8192) TT = 8192;
