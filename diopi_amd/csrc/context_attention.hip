@@ -33,6 +33,7 @@
 // second output.  That form is a template flag (GEN): the lightllm operator keeps its literal scale and its
 // compile-time causal structure.
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -48,6 +49,9 @@ constexpr int kHD = 128;   // head size of the MFMA kernel
 constexpr int kLD = kHD + 8;  // row pitch of the output tile in LDS, in elements (272 bytes: 16-byte aligned)
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 constexpr float kLazyLog2 = 8.0f;  // how far (in powers of two) the softmax reference maximum may lag behind
+// The same for the pipelined kernel's main loop, which pays for a move of the reference with the rest of the wave's tiles at
+// the plain loop's speed: probabilities up to 2^14 still fit the 16-bit types with full relative precision.
+constexpr float kPipeLazyLog2 = 14.0f;
 
 struct CtxArgs {
     const void* bStartLoc;
@@ -548,6 +552,477 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnMfma(T* 
     }
 }
 
+// v_mfma_f32_32x32x16 written out, accumulating in place.  The compiler does not see a matrix instruction in it, so it
+// inserts none of the wait states a read of the result by a vector instruction needs shortly after (11 for this 8-pass
+// shape); mfmaSettle() provides them where such a read follows within a few instructions.  In return the accumulators
+// stay where they are: with the builtin, a path that rewrites accumulators (the rare move of the softmax reference) made
+// the compiler settle the two paths' registers with a copy of every accumulator on the common path.
+template <typename T>
+struct MfmaInPlace;
+template <>
+struct MfmaInPlace<half_t> {
+    static __device__ __forceinline__ void acc(f32x16& c, u32x4 a, f16x8 b) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void start(f32x16& d, u32x4 a, f16x8 b, const f32x16& c) {
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+    }
+};
+template <>
+struct MfmaInPlace<bf16_t> {
+    static __device__ __forceinline__ void acc(f32x16& c, u32x4 a, bf16x8 b) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+    }
+    static __device__ __forceinline__ void start(f32x16& d, u32x4 a, bf16x8 b, const f32x16& c) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+    }
+};
+__device__ __forceinline__ void mfmaSettle() { asm volatile("s_nop 7\n\ts_nop 3" ::: "memory"); }
+
+// The lightllm prefill operator as one software-pipelined instruction stream per wave (fp16 / bf16, D == 128, causal).
+//
+// What the hardware does (measured): a matrix instruction keeps the SIMD's vector issue port for about 8 clocks whatever
+// its shape, and one that waits for the matrix pipe holds the port until it is issued.  Two waves that alternate between
+// blocks of products and blocks of vector work therefore do not overlap them, the blocks add up; and the 16x16x32 shape,
+// with twice the instructions per flop, leaves too little of the port for the softmax.  So: v_mfma_f32_32x32x16 (32
+// clocks of pipe, about 24 of them free for vector instructions), and every product is followed at once by its share of
+// the vector work of ANOTHER half tile, a few instructions that depend on nothing recent, so that the next product
+// arrives about when the pipe frees.  A key tile of 64 rows is handled as two halves of 32 keys; with (jt, h) the half h
+// of tile jt, one trip of the loop is
+//   phase 1:  S^T(jt, 1) = K . Q^T        8 products, between them the 16 exponentials and 8 packed conversions of (jt, 0)
+//   phase 2:  O^T += V^T(jt, 0) . P^T      8 products, between them the row sums of (jt, 0) and the maximum of (jt, 1)
+//   phase 3:  S^T(jt + 1, 0)               ... and the exponentials of (jt, 1)
+//   phase 4:  O^T += V^T(jt, 1) . P^T      ... and the row sums of (jt, 1), the maximum of (jt + 1, 0)
+// The K tile runs half a tile ahead of the V tile in LDS (two buffers each).  The last tile of a wave, the one its
+// diagonal crosses, is masked and finished outside the pipeline, and so is everything after a move of the softmax
+// reference (rare: see kPipeLazyLog2).  Layouts as in ctxAttnMfma: a lane owns query row lane % 32.
+template <typename T, int NWV>
+__global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k,
+                                                                               const T* __restrict__ v, CtxArgs a) {
+    constexpr float kScaleLog2 = 0.12751743082459868f;  // log2(e) / sqrt(128)
+    using Ops = MfmaInPlace<T>;
+    using Sum = Mfma32<T>;
+    using Frag = typename Mfma32<T>::Frag;
+    constexpr int BM = NWV * 32;
+    constexpr int kKRing = 3, kVRing = 3;  // operand fragments in registers: read-ahead = ring - 1 products
+    extern __shared__ __attribute__((aligned(16))) unsigned char dynSmem[];
+    T* smem = reinterpret_cast<T*>(dynSmem);
+
+    const int perXcd = (a.totalItems + kNumXcd - 1) / kNumXcd;
+    const int item = (blockIdx.x % kNumXcd) * perXcd + blockIdx.x / kNumXcd;
+    if (item >= a.totalItems) return;
+    const int head = item / a.tilesBound;
+    const int4 planned = a.plan[item % a.tilesBound];
+    if (planned.x < 0) return;
+    const int qt = __builtin_amdgcn_readfirstlane(planned.y);
+    const int64_t seqStart = __builtin_amdgcn_readfirstlane(planned.z);
+    const int L = __builtin_amdgcn_readfirstlane(planned.w);
+    const int m0 = qt * BM;
+
+    const int tid = threadIdx.x;
+    const int lane = tid % kWave;
+    const int wave = tid / kWave;
+    const int n = lane % 32;   // query column of this lane in every accumulator
+    const int hh = lane / 32;  // which half of the k slots / which 4-row sub-block of the accumulator
+    const int64_t qPitch = static_cast<int64_t>(a.H) * kHD;
+    const T* qBase = q + seqStart * qPitch + static_cast<int64_t>(head) * kHD;
+    const T* kBase = k + seqStart * qPitch + static_cast<int64_t>(head) * kHD;
+    const T* vBase = v + seqStart * qPitch + static_cast<int64_t>(head) * kHD;
+
+    // ---- Q^T fragments (B operand of the first product): query row n, dims 16 st + 8 hh .. + 7, scaled by
+    // log2(e) / sqrt(D) and rounded to the element type once (see ctxAttnMfma) ----
+    Frag qf[kHD / 16];
+    {
+        const int row = m0 + wave * 32 + n;
+        const int rowLd = row < L ? row : L - 1;
+#pragma unroll
+        for (int st = 0; st < kHD / 16; ++st) {
+            FragBits<Frag> u;
+            u.raw = *reinterpret_cast<const u32x4*>(qBase + rowLd * qPitch + st * 16 + hh * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[st][e] = static_cast<T>(static_cast<float>(u.f[e]) * kScaleLog2);
+        }
+    }
+
+    f32x16 o[kHD / 32];
+#pragma unroll
+    for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[mb][r] = 0.f;
+    }
+    f32x16 s0, s1;     // scores of the lower / upper 32 keys of a tile: register r is key 8 (r / 4) + 4 hh + r % 4
+    float lRun = 0.f;  // this lane's share of the row sum (the other half lives in lane ^ 32)
+    // minus the reference maximum of the lane's query row (in powers of two), as the accumulator the first product of a
+    // half starts from: the scores arrive as score - reference, ready for the exponential
+    f32x16 negRef;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negRef[r] = 0.f;
+    Frag pf[2];        // probabilities of one half, per group of 16 keys
+
+    const int kEnd = m0 + BM < L ? m0 + BM : L;
+    const int numKeyTiles = (kEnd + kBN - 1) / kBN;
+
+    // ---- tile staging (see ctxAttnMfma): K tile c in buffer c & 1 at 32 KiB * (c & 1), V tile c of buffer c & 1 16 KiB behind it ----
+    constexpr int kTileBytes = kBN * kHD * static_cast<int>(sizeof(T));
+    constexpr int kChunks = kBN / 4 / NWV;
+    using LdsByte = __attribute__((address_space(3))) unsigned char;
+    LdsByte* const lds = (LdsByte*)dynSmem;
+    const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const int waveU = __builtin_amdgcn_readfirstlane(wave);
+    const int waveRowLo = m0 + waveU * 32;
+    const bool active = waveRowLo < L;
+    const int dg = waveRowLo / kBN;  // the tile this wave's diagonal crosses, its last one
+    const int rowBytes = static_cast<int>(qPitch) * static_cast<int>(sizeof(T));
+    int kSrc[kChunks], vSrc[kChunks];
+#pragma unroll
+    for (int it = 0; it < kChunks; ++it) {
+        const int r = (waveU * kChunks + it) * 4 + lane / 16;
+        kSrc[it] = r * rowBytes + (((lane % 16) ^ (r & 15)) * 16);
+        vSrc[it] = r * rowBytes + (((lane % 16) ^ (4 * (r & 3))) * 16);
+    }
+    // The K tiles are cut half a tile off the V tiles: K tile c holds key rows 64 c - 32 .. 64 c + 31, because one trip of
+    // the loop multiplies by the upper half of one 64-key tile and the lower half of the next, and a buffer can only be
+    // refilled once every wave has left it.  K tile 0 therefore has no lower half (nothing is fetched for it), and there
+    // is one K tile more than V tiles.  Rows past the sequence are outside the tile's buffer descriptor and arrive as zeros.
+    const int64_t tileStride = static_cast<int64_t>(kBN) * qPitch * static_cast<int64_t>(sizeof(T));
+    // the tile addresses live in scalar registers (the sequence's first row came from memory, into a vector register)
+    uint64_t kNext = reinterpret_cast<uint64_t>(uniformPointer(kBase)) - static_cast<uint64_t>(tileStride / 2);
+    uint64_t vNext = reinterpret_cast<uint64_t>(uniformPointer(vBase));
+    uint32_t kDst = ldsBase + waveU * kChunks * 1024, vDst = ldsBase + kTileBytes + waveU * kChunks * 1024;
+    int kRow = -kBN / 2, vRow = 0;  // first sequence row of the next tile to request
+    auto request = [&](uint64_t& next, uint32_t& dst, int& row, const int (&src)[kChunks]) {
+        const int valid = L - row < kBN ? L - row : kBN;  // rows of the tile inside the sequence
+        if (valid > 0 && row < kEnd) {
+            const uint32_t bytes = static_cast<uint32_t>(((valid - 1) * qPitch + kHD) * static_cast<int64_t>(sizeof(T)));
+            const u32x4 buf = {static_cast<uint32_t>(next), static_cast<uint32_t>(next >> 32) & 0xffffu, bytes, kRawBufferWord3};
+#pragma unroll
+            for (int it = 0; it < kChunks; ++it) {
+                if (row >= 0 || (waveU * kChunks + it) * 4 >= kBN / 2) loadToLds16(buf, dst + it * 1024, src[it]);
+            }
+        }
+        next += tileStride;
+        dst ^= 2 * kTileBytes;
+        row += kBN;
+    };
+
+    // ---- operand addresses (LDS addresses, the staging area's own included) ----
+    // K (A operand of the first product), step st of half h: row 32 h + n, packet 2 st + hh, swizzled by the row.
+    // V^T (A operand of the second), block mb, key group u of half h: two transposing reads (see ctxAttnMfma); in each,
+    // the lane supplies the address of 4 dims of key row 32 h + 16 u + 8 w + 4 hh + (lane % 16) / 4.
+    // The step / block index enters through the swizzle's exclusive-or, on bits the lane's part also uses, so it cannot
+    // ride in the instruction's offset field: one register per st and per mb.  They point into the buffers of the tile
+    // at hand and change buffers by flipping one bit, once per tile.
+    uint32_t kAddr[kHD / 16], vAddr[kHD / 32];
+    {
+        const int hx = hh ^ (n & 15);
+#pragma unroll
+        for (int st = 0; st < kHD / 16; ++st) kAddr[st] = ldsBase + n * 256 + (((2 * st) ^ hx) * 16);
+        const int g16 = lane / 16, kk = (lane % 16) / 4, qq = lane % 4;
+        const int cLo = 2 * (g16 % 2) + qq / 2;
+#pragma unroll
+        for (int mb = 0; mb < kHD / 32; ++mb) vAddr[mb] = ldsBase + kTileBytes + (4 * hh + kk) * 256 + ((4 * (mb ^ kk) + cLo) * 16) + (qq % 2) * 8;
+    }
+    // The query fragments must have arrived before the first tile request: a wait for them after it would also wait for
+    // the request, which the compiler does not count.
+#pragma unroll
+    for (int st = 0; st < kHD / 16; ++st) asm volatile("" : "+v"(qf[st]));
+
+    using LdsVec = const __attribute__((address_space(3))) u32x4*;
+    using LdsQuad = __attribute__((address_space(3))) s16x4*;
+    auto readK = [&](int h, int st) -> u32x4 {  // rows 32 h .. 32 h + 31 of the K tile kAddr points at
+        return *reinterpret_cast<LdsVec>(static_cast<uintptr_t>(kAddr[st] + h * 32 * 256));
+    };
+    auto readV = [&](int h, int f) -> u32x4 {  // fragment f = 4 u + mb of half h of the V tile vAddr points at
+        const uintptr_t base = vAddr[f % 4] + (h * 32 + (f / 4) * 16) * 256;
+        const s16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsQuad>(base));
+        const s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsQuad>(base + 8 * 256));
+        u32x4 r;
+        r[0] = __builtin_bit_cast(u32x2, t0)[0];
+        r[1] = __builtin_bit_cast(u32x2, t0)[1];
+        r[2] = __builtin_bit_cast(u32x2, t1)[0];
+        r[3] = __builtin_bit_cast(u32x2, t1)[1];
+        return r;
+    };
+    auto flipK = [&]() {
+#pragma unroll
+        for (int st = 0; st < kHD / 16; ++st) kAddr[st] ^= 2 * kTileBytes;
+    };
+    auto flipV = [&]() {
+#pragma unroll
+        for (int mb = 0; mb < kHD / 32; ++mb) vAddr[mb] ^= 2 * kTileBytes;
+    };
+
+    // exponential of score r of a half; packing of two of them into word w (= r / 2) of the probability fragments
+    auto expOne = [&](const f32x16& s, int r) -> float {
+        return __builtin_amdgcn_exp2f(s[r]);
+    };
+    auto packPair = [&](int w, float e0, float e1) -> uint32_t {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef T tx2 __attribute__((ext_vector_type(2)));
+        const uint32_t word = __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{e0, e1}), tx2));  // one packed conversion
+        FragBits<Frag> u;
+        u.f = pf[w / 4];
+        u.raw[w % 4] = word;
+        pf[w / 4] = u.f;
+        return word;
+    };
+    // this lane's maximum over the 16 keys it holds of a half, as a chain of 8 instructions; step i of it
+    auto maxStep = [&](const f32x16& s, int i, float m) -> float {
+        if (i == 0) return max3(s[0], s[1], s[2]);
+        if (i == 7) return max3(m, s[15], s[15]);
+        return max3(m, s[2 * i + 1], s[2 * i + 2]);
+    };
+    // Moves the reference of the lane's query row up by `up`: scales what has been accumulated, shifts the scores of the
+    // half at hand.  Rarely taken.
+    auto rescale = [&](f32x16& s, float up) {
+        const float alpha = __builtin_amdgcn_exp2f(-up);
+        lRun *= alpha;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) negRef[r] -= up;
+#pragma unroll
+        for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[mb][r] *= alpha;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] -= up;
+    };
+
+    // S^T of the 32 keys in rows 32 h .. of the K tile kAddr points at, into sN, with the exponentials of half sC dealt out
+    // between the products (EXP) or nothing in between.
+    auto scores = [&](auto expTag, int h, f32x16& sN, const f32x16& sC, const float (&early)[8]) {
+        constexpr bool EXP = decltype(expTag)::value;
+        u32x4 kf[kKRing];
+        float late[8];  // exponentials of scores 8..15, one per step
+#pragma unroll
+        for (int t = 0; t < kKRing - 1; ++t) kf[t] = readK(h, t);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            if (t + kKRing - 1 < 8) kf[(t + kKRing - 1) % kKRing] = readK(h, t + kKRing - 1);
+            if (t == 0) {
+                Ops::start(sN, kf[0], qf[0], negRef);
+            } else {
+                Ops::acc(sN, kf[t % kKRing], qf[t]);
+            }
+            if constexpr (EXP) {
+                // one exponential and one packed conversion per product; scores 0..7 were exponentiated during the
+                // products of the phase before (`early`), and a pair is packed two or more steps after its exponentials
+                late[t] = expOne(sC, 8 + t);
+                if (t < 4) {
+                    packPair(t, early[2 * t], early[2 * t + 1]);
+                } else if (t < 7) {
+                    packPair(t, late[2 * (t - 4)], late[2 * (t - 4) + 1]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (EXP) {
+            packPair(7, late[6], late[7]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // O^T += V^T(half h of the tile vAddr points at) . P^T; dealt out between the products (MAX): the row sums of the
+    // probabilities at hand and the lane maximum of half sN (returned in tm)
+    auto values = [&](auto maxTag, int h, const f32x16& sN, float& tm, float (&early)[8]) {
+        constexpr bool MAX = decltype(maxTag)::value;
+        u32x4 vf[kVRing];
+#pragma unroll
+        for (int f = 0; f < kVRing - 1; ++f) vf[f] = readV(h, f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < 8; ++f) {
+            if (f + kVRing - 1 < 8) vf[(f + kVRing - 1) % kVRing] = readV(h, f + kVRing - 1);
+            Ops::acc(o[f % 4], vf[f % kVRing], pf[f / 4]);
+            if constexpr (MAX) {
+                FragBits<Frag> u;
+                u.f = pf[f / 4];
+                lRun = Sum::addPair(u.raw[f % 4], lRun);
+                // (a product behind: the scores come from matrix instructions the compiler does not see, and a vector
+                // instruction may read them only a dozen wait states later)
+                if (f >= 1) tm = maxStep(sN, f - 1, tm);
+                // the first eight exponentials of the half whose maximum is being taken: should the maximum turn out too
+                // high they are thrown away with the rest of the pipeline's state
+                if (f >= 1) early[f - 1] = expOne(sN, f - 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (MAX) {
+            tm = maxStep(sN, 7, tm);
+            early[7] = expOne(sN, 7);
+        }
+    };
+    // exponentials of half s into pf, row sums: the unpipelined form
+    auto probabilities = [&](const f32x16& s) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) lRun = Sum::addPair(packPair(w, expOne(s, 2 * w), expOne(s, 2 * w + 1)), lRun);
+    };
+    using Yes = std::true_type;
+    using No = std::false_type;
+
+    // K tile jt + 1 and V tile jt have landed, every wave has left K tile jt and V tile jt - 1: their buffers take the next ones
+    auto top = [&]() {
+        waitLdsLoads();
+        __syncthreads();
+        request(kNext, kDst, kRow, kSrc);
+        request(vNext, vDst, vRow, vSrc);
+    };
+
+    // ---- prologue: K tile 0; then K tile 1 and V tile 0 travel while the scores of the first 32 keys are computed ----
+    request(kNext, kDst, kRow, kSrc);
+    waitLdsLoads();
+    __syncthreads();
+    request(kNext, kDst, kRow, kSrc);
+    request(vNext, vDst, vRow, vSrc);
+    float tm = 0.f;
+    float early[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // exponentials of scores 0..7 of the half that is next in line
+    if (active) {
+        scores(No(), 1, s0, s0, early);
+        mfmaSettle();
+        if (dg > 0) {  // the first half sets the reference
+            float m = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) m = maxStep(s0, i, m);
+            rescale(s0, maxWithOtherHalf(m));
+#pragma unroll
+            for (int r = 0; r < 8; ++r) early[r] = expOne(s0, r);
+        }
+    }
+    flipK();  // from here on kAddr points at K tile jt + 1
+    int jt = 0;
+    if (active) {
+        // A phase that finds the reference too low for some row leaves the pipeline for good: the rest of the wave's
+        // tiles go through the plain loop below, which moves the reference where it has to.  With the threshold at
+        // 2^kPipeLazyLog2 above the maximum of the wave's first 32 keys that is rare, and the pipelined loop keeps no
+        // path on which accumulators are rewritten.  One exit, at the bottom, and the second half of a trip under a
+        // condition: with several exits the compiler's loop-exit unification hands every live value through blocks of
+        // register copies.
+        auto tooLow = [&]() -> bool { return __any(tm > kPipeLazyLog2); };
+        int event = 0;
+        if (jt < dg) {
+            do {
+                top();
+                scores(Yes(), 0, s1, s0, early);  // phase 1
+                values(Yes(), 0, s1, tm, early);  // phase 2
+                if (tooLow()) {
+                    event = 1;
+                } else {
+                    scores(Yes(), 1, s0, s1, early);  // phase 3
+                    values(Yes(), 1, s0, tm, early);  // phase 4
+                    flipK();
+                    flipV();
+                    ++jt;
+                    // the unmasked maximum of the diagonal tile must not move the reference: its turn comes below
+                    if (jt < dg && tooLow()) event = 2;
+                }
+            } while (jt < dg && event == 0);
+        }
+        // the row's maximum over the 32 keys of half s; moves the reference when it is more than the lazy margin above it
+        auto settleHalf = [&](f32x16& s) {
+            mfmaSettle();
+            float m = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) m = maxStep(s, i, m);
+            if (__any(m > kLazyLog2)) rescale(s, fmaxf(maxWithOtherHalf(m), 0.f));
+        };
+        float unused = 0.f;
+        float unusedEarly[8];
+        if (event == 1) {  // the upper half of tile jt is still to do
+            settleHalf(s1);
+            probabilities(s1);
+            values(No(), 1, s1, unused, unusedEarly);
+            scores(No(), 1, s0, s0, unusedEarly);
+            flipK();
+            flipV();
+            ++jt;
+        }
+        if (event != 0) {
+            while (jt < dg) {  // s0 holds the lower half of tile jt, not yet looked at
+                top();
+                settleHalf(s0);
+                probabilities(s0);
+                values(No(), 0, s0, unused, unusedEarly);
+                scores(No(), 0, s1, s1, unusedEarly);
+                settleHalf(s1);
+                probabilities(s1);
+                values(No(), 1, s1, unused, unusedEarly);
+                scores(No(), 1, s0, s0, unusedEarly);
+                flipK();
+                flipV();
+                ++jt;
+            }
+        }
+        // ---- the diagonal tile: mask, maximum, exponentials, second product, nothing overlapped.  A wave whose rows are
+        // the lower 32 of its tile's 64 sees only the lower half of the keys. ----
+        top();
+        const bool both = (waveRowLo & 32) != 0;
+        if (both) scores(No(), 0, s1, s1, unusedEarly);
+        mfmaSettle();  // also for the accumulators of the loop's last products
+        const int key0 = dg * kBN;
+        const int row = waveRowLo + n;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = key0 + 8 * (r / 4) + 4 * hh + r % 4;
+            if (key > row) s0[r] = -1e30f;
+            if (!both || key + 32 > row) s1[r] = -1e30f;
+        }
+        float m = 0.f, m1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            m = maxStep(s0, i, m);
+            m1 = maxStep(s1, i, m1);
+        }
+        float up = maxWithOtherHalf(fmaxf(m, m1));
+        const bool first = dg == 0;
+        if (first || __any(up > kLazyLog2)) {
+            if (!first) up = fmaxf(up, 0.f);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s1[r] -= up;
+            rescale(s0, up);
+        }
+        probabilities(s0);
+        values(No(), 0, s0, unused, unusedEarly);
+        if (both) {
+            probabilities(s1);
+            values(No(), 1, s1, unused, unusedEarly);
+        }
+        ++jt;
+    }
+    mfmaSettle();
+    for (; jt < numKeyTiles; ++jt) top();  // the other waves' remaining tiles: this wave only fetches its share
+
+    // ---- normalise, transpose through LDS, write rows with 16-byte stores ----
+    const float lTot = lRun + __shfl_xor(lRun, 32, kWave);
+    const float inv = 1.0f / lTot;
+    waitLdsLoads();
+    __syncthreads();  // the K/V tiles are dead and no request is in flight; reuse the storage as a [BM][kLD] output tile
+    T* sO = smem;
+#pragma unroll
+    for (int mb = 0; mb < kHD / 32; ++mb) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+            // registers 4 rq .. 4 rq + 3 of o[mb] are dims 32 mb + 8 rq + 4 hh .. + 3
+            T pk[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = static_cast<T>(o[mb][4 * rq + e] * inv);
+            *reinterpret_cast<u32x2*>(sO + (wave * 32 + n) * kLD + 32 * mb + 8 * rq + 4 * hh) = *reinterpret_cast<const u32x2*>(pk);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    T* oBase = out + seqStart * qPitch + static_cast<int64_t>(head) * kHD;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int id = it * kWave + lane;
+        const int row = id / 16;
+        const int c = id % 16;
+        const int grow = m0 + wave * 32 + row;
+        if (grow < L) {
+            const u32x4 val = *reinterpret_cast<const u32x4*>(sO + (wave * 32 + row) * kLD + c * 8);
+            *reinterpret_cast<u32x4*>(oBase + grow * qPitch + c * 8) = val;
+        }
+    }
+}
+
 // Any dtype / head size up to 512: one wave per (query row, head); lanes split the head dimension.
 template <typename T, typename AccT>
 __global__ __launch_bounds__(kWave) void ctxAttnGeneric(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, CtxArgs a,
@@ -636,6 +1111,13 @@ diopiError_t launchMfma(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     constexpr int kStaging = 2 * 2 * kBN * kHD, kOutTile = BM * kLD;  // elements: two (K, V) buffers; the output tile that reuses them
     constexpr int ldsBytes = (kStaging > kOutTile ? kStaging : kOutTile) * static_cast<int>(sizeof(T));
     ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(ctxAttnMfma<T, NWV, GEN>), ldsBytes));
+    if constexpr (!GEN) {  // the lightllm operator: causal, one key/value head per query head, the literal scale
+        ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(ctxAttnPipe<T, NWV>), ldsBytes));
+        hipLaunchKernelGGL((ctxAttnPipe<T, NWV>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q),
+                           static_cast<const T*>(k), static_cast<const T*>(v), a);
+        ROCM_LAUNCH_CHECK();
+        return diopiSuccess;
+    }
     hipLaunchKernelGGL((ctxAttnMfma<T, NWV, GEN>), dim3(grid), dim3(NWV * kWave), ldsBytes, stream, static_cast<T*>(out), static_cast<const T*>(q),
                        static_cast<const T*>(k), static_cast<const T*>(v), a);
     ROCM_LAUNCH_CHECK();

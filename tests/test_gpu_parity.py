@@ -838,6 +838,41 @@ def test_context_attention_long_odd_lengths_whole_output():
                       f"two long sequences {dt}")
 
 
+def _rising_case(L, H, dt, profile, what):
+    """Scores that climb along the sequence: q = a * u + noise, k_j = b_j * u + noise with u a unit vector, so that the
+    score of key j is about a * b_j (in powers of two after the softmax scale: `profile(j)`)."""
+    g = gen(604)
+    u = torch.ones(128) / math.sqrt(128.0)
+    a = 8.0
+    to_raw = math.sqrt(128.0) / math.log2(math.e)  # from powers of two to the unscaled dot product
+    b = torch.tensor([profile(j) * to_raw / a for j in range(L)])
+    q = (a * u + 0.05 * torch.randn(L, H, 128, generator=g)).to(dt).to(DEV)
+    k = (b.reshape(L, 1, 1) * u + 0.05 * torch.randn(L, H, 128, generator=g)).to(dt).to(DEV)
+    v = torch.randn(L, H, 128, generator=g).to(dt).to(DEV)
+    bs = torch.tensor([0], dtype=torch.int32, device=DEV)
+    bl = torch.tensor([L], dtype=torch.int32, device=DEV)
+    out = torch.full_like(q, 77.0)
+    F.context_attention(q, k, v, out, bs, bl, L)
+    ex = torch.full(q.shape, 77.0, dtype=torch.float64)
+    O.context_attention(q.cpu(), k.cpu(), v.cpu(), ex, bs.cpu(), bl.cpu(), L, exact=True)
+    assert bool(torch.isfinite(out.float()).all()), what + ": non-finite output"
+    assert_close(out.cpu(), ex, what=what + " vs float64", **TOL[dt])
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_context_attention_rising_scores_move_the_softmax_reference(dtype):
+    # The prefill kernels keep a lazily updated reference maximum per query row; seeded normal tensors never move it after
+    # the first keys.  Here the scores climb by 2^60 along the sequence, steadily (the reference moves every few tiles) or
+    # in single jumps that land in the lower and in the upper half of a 64-key tile, early and late in a query tile's keys.
+    dt = TORCH_DTYPES[dtype]
+    for L in (700, 1100):  # 128-row and 256-row query tiles
+        _rising_case(L, 2, dt, lambda j: 60.0 * j / L, f"steady climb L={L} {dtype}")
+        _rising_case(L, 2, dt, lambda j: (40.0 if j >= 100 else 0.0), f"jump at key 100 (upper half of tile 1) L={L} {dtype}")
+        _rising_case(L, 2, dt, lambda j: (40.0 if j >= 200 else 0.0) + (30.0 if j >= 457 else 0.0),
+                     f"jumps at keys 200 (lower half of tile 3) and 457 L={L} {dtype}")
+        _rising_case(L, 2, dt, lambda j: 30.0 * (j % 64 == 63) + 20.0 * (j // 64), f"staircase with spikes L={L} {dtype}")
+
+
 def test_context_attention_config4_scaled():
     w = W.cfg4(DEV, seed=4, scale=0.125)  # 8 sequences of 128..512 tokens
     _context_case(w["q"], w["k"], w["v"], w["b_start_loc"], w["b_seq_len"], w["max_input_len"], torch.float16, "cfg4 x 1/8")
