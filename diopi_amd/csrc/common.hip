@@ -278,21 +278,6 @@ diopiError_t grantDynamicLds(const void* kernel, int bytes) {
     return diopiSuccess;
 }
 
-int envInt(const char* name, int fallback) {
-    // what is remembered is the environment (set or not, and to what), never a caller's fallback: fallbacks depend
-    // on the shapes of the call at hand
-    static std::mutex mtx;
-    static std::map<std::string, std::pair<bool, int>> cache;
-    std::lock_guard<std::mutex> lock(mtx);
-    auto it = cache.find(name);
-    if (it == cache.end()) {
-        const char* s = std::getenv(name);
-        const bool set = s != nullptr && *s != '\0';
-        it = cache.emplace(name, std::make_pair(set, set ? std::atoi(s) : 0)).first;
-    }
-    return it->second.first ? it->second.second : fallback;
-}
-
 }  // namespace rocm
 
 // ---- library identification (reference: impl/torch/functions/functions.cpp:37-66) ----

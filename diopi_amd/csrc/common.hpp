@@ -120,10 +120,6 @@ const DeviceInfo& deviceInfo();
 // to the device the call runs on; a process may hold several).
 diopiError_t grantDynamicLds(const void* kernel, int bytes);
 
-// Integer knob from the environment, for tuning experiments: the variable is looked up once per name; when it is unset
-// every call gets its own fallback (fallbacks depend on the shapes of the call at hand).
-int envInt(const char* name, int fallback);
-
 inline int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 }  // namespace rocm

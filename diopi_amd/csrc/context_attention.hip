@@ -1148,9 +1148,9 @@ diopiError_t dispatchAttention(diopiContextHandle_t ctx, hipStream_t stream, con
     const bool planFits = (4 * static_cast<int64_t>(a.batch) + a.rows / kBMMin + 1) * 4 <= 64 * 1024 && a.rows <= INT32_MAX;
     // the tile requests address a 64-row tile with 32-bit byte offsets
     const bool tileFits = static_cast<int64_t>(a.H) * kHD * 8 * kBN < INT32_MAX;
-    const bool fast = D == kHD && aligned && planFits && tileFits && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    const bool fast = D == kHD && aligned && planFits && tileFits;
     // 256-row query tiles (8 waves share each K/V tile) once the sequences are long enough to fill them
-    const bool wide = envInt("DIOPI_ROCM_CTX_WAVES", a.rows >= 1024 * static_cast<int64_t>(a.batch) ? 8 : 4) == 8;
+    const bool wide = a.rows >= 1024 * static_cast<int64_t>(a.batch);
     switch (vQ.dtype) {
         case diopi_dtype_float16:
             return fast ? (wide ? launchMfma<half_t, 8, GEN>(ctx, stream, vOut.data, vQ.data, vK.data, vV.data, a, store)

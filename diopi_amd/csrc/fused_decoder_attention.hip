@@ -653,8 +653,8 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     // max_seq_len.  Measured at 64 rows of 512..2047 tokens, 32 kv heads, items taken longest first: 1024 tokens per range
     // 237-238 us per call in two harnesses, 512: 247-251, 2048 (no partials, no merge launch): 235 in one, 254 in the other
     AttnSplit sp;
-    sp.TT = envInt("DIOPI_ROCM_FUSEDDEC_TT", 1024);
-    sp.TT = static_cast<int>(ceilDiv(sp.TT, kAttnStep)) * kAttnStep;
+    sp.TT = 1024;
+    static_assert(1024 % kAttnStep == 0, "a range is a whole number of steps");
     sp.splits = static_cast<int>(ceilDiv(max_seq_len, sp.TT));
     sp.partAcc = nullptr;
     sp.partMl = nullptr;
@@ -675,7 +675,6 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
         // their head: 33.2 us at 96 heads x 4096 against 35.6 us for 256 runs that cross heads); otherwise equal runs
         int64_t wgs = std::max<int64_t>(1, deviceInfo().numCU / rowBlocks);
         if (pl.tiles <= wgs) wgs = pl.tiles * std::min<int64_t>(wgs / pl.tiles, ceilDiv(pl.stepsPerTile, kProjWaves));
-        wgs = envInt("DIOPI_ROCM_FUSEDDEC_WGS", static_cast<int>(wgs));
         wgs = std::max<int64_t>(1, std::min<int64_t>(wgs, ceilDiv(units, kProjWaves)));
         pl.unitsPerWg = static_cast<int>(ceilDiv(units, wgs));
         if (pl.tiles <= wgs && pl.stepsPerTile % pl.unitsPerWg != 0 && pl.unitsPerWg < pl.stepsPerTile)

@@ -575,11 +575,10 @@ diopiError_t launchFwdFast(hipStream_t stream, const TensorView& out, const Tens
     if (sizeof(TOut) != sizeof(TIn) && (reinterpret_cast<uintptr_t>(out.data) & 7) != 0) return diopiSuccess;
     const float feps = static_cast<float>(eps);
     const int n2 = static_cast<int>(d.n2);
-    if (nvec > 2 * kWave && envInt("DIOPI_ROCM_RMSFWD_WAVEROW", 0) == 0) {
+    if (nvec > 2 * kWave) {
         // long rows: one 256-thread group per run of rows
         const int nvt = static_cast<int>(ceilDiv(nvec, kFwdThreads));
-        int rpb = envInt("DIOPI_ROCM_RMSFWD_ROWS_PER_BLOCK", 1);
-        if (rpb < 1) rpb = 1;
+        const int rpb = 1;  // rows per work-group
         const unsigned gridB = static_cast<unsigned>(ceilDiv(d.n1, rpb));
 #define ROCM_FWDB_CASE(NVC)                                                                                                                         \
     if (bias != nullptr) {                                                                                                                          \
@@ -690,7 +689,7 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
     const int groups = gBias ? 2 : 4;
     // one work-group per compute unit (fewer when there are not enough rows to give every team one)
-    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * envInt("DIOPI_ROCM_RMSBWD_BLOCKS_PER_CU", 1);
+    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU);
     const int numParts = static_cast<int>(std::min<int64_t>(maxBlocks, ceilDiv(d.n1, groups)));
     const int n2 = static_cast<int>(d.n2);
     const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(ColAcc);

@@ -96,7 +96,7 @@ diopiError_t launchV2(hipStream_t stream, const TensorView& q, const TensorView&
     const int half = dim / 2;
     const bool aligned = ((reinterpret_cast<uintptr_t>(q.data) | reinterpret_cast<uintptr_t>(k.data) | reinterpret_cast<uintptr_t>(c.data) |
                            reinterpret_cast<uintptr_t>(s.data)) & 15) == 0;
-    if (aligned && half % EPV == 0 && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0) {
+    if (aligned && half % EPV == 0) {
         const int packetsPerHalf = half / EPV;
         const int headChunks = static_cast<int>(ceilDiv(hq + hk, kRot2HeadsPerLane));
         const int64_t items = tokens * headChunks * packetsPerHalf;

@@ -200,9 +200,6 @@ __global__ __launch_bounds__(kAttThreads) void tokenAttStaged(T* __restrict__ ou
     if (order == 1) {  // y = tile, z = sequence: the tiles of a sequence one after the other
         i = static_cast<int>(blockIdx.z);
         tileIdx = static_cast<int>(blockIdx.y);
-    } else if (order == 3) {  // y = sequence, z = tile
-        i = static_cast<int>(blockIdx.y);
-        tileIdx = static_cast<int>(blockIdx.z);
     } else {  // y = sequence, z = tile, the sequence rotated by the tile index: consecutive work-groups mix tiles of different sequences
         i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
         tileIdx = static_cast<int>(blockIdx.z);
@@ -378,17 +375,12 @@ template <typename T>
 diopiError_t launchMfma(hipStream_t stream, void* out, const void* q, const void* k, const DecodeArgs& a, float scale) {
     constexpr int TT = 128;
     // kv heads per work-group: about 256 KiB of K per group, at least one head per wave
-    int HB = a.Hkv < 8 ? a.Hkv : 8;
-    HB = envInt("DIOPI_ROCM_TOKATT_HB", HB);
+    const int HB = a.Hkv < 8 ? a.Hkv : 8;
     ROCM_CHECK(a.batch <= 65535 && ceilDiv(a.maxInputLen, TT) <= 65535, "batch %d / max_input_len %d exceed the launch limits (65535 sequences, 65535 tiles of %d tokens)", a.batch, a.maxInputLen, static_cast<int>(TT));
     const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HB)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
-    if (a.D == 128) {
-        hipLaunchKernelGGL((tokenAttMfma<T, 4, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
-                           static_cast<const T*>(k), a, HB, scale);
-    } else {
-        hipLaunchKernelGGL((tokenAttMfma<T, 2, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
-                           static_cast<const T*>(k), a, HB, scale);
-    }
+    // head size 64 (128 goes through the staged kernel)
+    hipLaunchKernelGGL((tokenAttMfma<T, 2, TT>), grid, dim3(kAttThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(q),
+                       static_cast<const T*>(k), a, HB, scale);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
@@ -398,20 +390,13 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     // heads per wave, head slots per work-group (waves beyond the head slots take other token units).  One head per
     // wave and short token tiles measured best once the head groups of a tile are dispatched next to each other:
     // neighbouring work-groups then stream neighbouring pieces of the same cache rows at the same time.
-    int HW = 1;
-    HW = envInt("DIOPI_ROCM_TOKATT_HW", HW);
-    if (HW != 1 && HW != 2 && HW != 4) HW = 1;
+    constexpr int HW = 1;
     const int slots = static_cast<int>(ceilDiv(a.Hkv, HW));
-    int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
-    HS = envInt("DIOPI_ROCM_TOKATT_HS", HS);
-    if (HS != 1 && HS != 2 && HS != 4) HS = 1;
+    const int HS = slots >= 4 ? 4 : (slots >= 2 ? 2 : 1);
     // tokens per work-group: with one query head per kv head, tiles of 64 tokens measured 1.7 % faster than 128 (64
     // sequences of 512..2048 tokens, 32 heads); with 8 query heads per kv head (128 sequences of 1024..8192 tokens, 8 kv
     // heads) 256 is 4 % faster than 128 and 512 is 1 % slower than 256: longer pieces of every logits row per write-out
-    int TT = envInt("DIOPI_ROCM_TOKATT_TT", a.G == 1 ? 64 : 256);
-    TT = TT / 64 * 64;
-    if (TT < 64) TT = 64;
-    if (TT > 1024) TT = 1024;
+    int TT = a.G == 1 ? 64 : 256;
     // the scores of a tile wait in LDS for the write-out: at most 40 KiB of them
     const int outRows = HS * HW * a.G;
     while (TT > 64 && outRows * (TT + 8) * static_cast<int>(sizeof(T)) > 40 * 1024) TT -= 64;
@@ -423,20 +408,11 @@ diopiError_t launchStaged(hipStream_t stream, void* out, const void* q, const vo
     // sequence would stay on a few XCDs and ragged lengths would unbalance them: y = sequence, z = tile, the sequence rotated by
     // the tile index (cfg5, 2 head groups: 242 us; unrotated 264, tiles in sequence order 268).
     const int gridX = static_cast<int>(ceilDiv(a.Hkv, HS * HW));
-    const int order = envInt("DIOPI_ROCM_TOKATT_ORDER", gridX % kNumXcd == 0 ? 1 : 0);
+    const int order = gridX % kNumXcd == 0 ? 1 : 0;
     const dim3 grid = order == 1 ? dim3(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)), static_cast<unsigned>(a.batch))
                                  : dim3(static_cast<unsigned>(ceilDiv(a.Hkv, HS * HW)), static_cast<unsigned>(a.batch), static_cast<unsigned>(ceilDiv(a.maxInputLen, TT)));
-#define ROCM_STAGED_CASE(HWC)                                                                                                                         \
-    hipLaunchKernelGGL((tokenAttStaged<T, HWC>), grid, dim3(kAttThreads), outLds, stream, static_cast<T*>(out), static_cast<const T*>(q),             \
-                       static_cast<const T*>(k), a, TT, HS, scale, order)
-    if (HW == 4) {
-        ROCM_STAGED_CASE(4);
-    } else if (HW == 2) {
-        ROCM_STAGED_CASE(2);
-    } else {
-        ROCM_STAGED_CASE(1);
-    }
-#undef ROCM_STAGED_CASE
+    hipLaunchKernelGGL((tokenAttStaged<T, HW>), grid, dim3(kAttThreads), outLds, stream, static_cast<T*>(out), static_cast<const T*>(q),
+                       static_cast<const T*>(k), a, TT, HS, scale, order);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
@@ -468,11 +444,10 @@ diopiError_t tokenAttention(diopiContextHandle_t ctx, const TensorView& vOut, co
 
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
-    const bool fast = (D == 128 || D == 64) && a.G <= 16 && ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data)) & 15) == 0 &&
-                      envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+    const bool fast = (D == 128 || D == 64) && a.G <= 16 && ((reinterpret_cast<uintptr_t>(vQ.data) | reinterpret_cast<uintptr_t>(vK.data)) & 15) == 0;
     // the element type's matmul rounds the fp32 dot to T, then the division by sqrt(D) rounds again
     const float scale = 1.0f / static_cast<float>(std::sqrt(static_cast<double>(D)));
-    const bool staged = fast && D == 128 && envInt("DIOPI_ROCM_TOKATT_DIRECT", 0) == 0;
+    const bool staged = fast && D == 128;
     switch (vQ.dtype) {
         case diopi_dtype_float16:
             if (staged) return launchStaged<half_t>(stream, vOut.data, vQ.data, vK.data, a, scale);

@@ -34,7 +34,6 @@ struct SplitArgs {
     float* partMl;   // [batch, splits, H, 2]  (running max, denominator)
     int splits;      // ranges per sequence the scratch is sized for
     int TT;          // tokens per range (multiple of kSub)
-    int headsPerGroup;  // kv heads a work-group streams side by side: 1, 2 or 4 (its waves are heads x sub-tile phases)
 };
 
 // Matrix-core kernel (16-bit types, D == 128, any G <= 16): per kv head the weighted sum is the small product
@@ -125,7 +124,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
     const int64_t t0 = static_cast<int64_t>(zIdx) * sp.TT;
-    const int HG = sp.headsPerGroup;
+    constexpr int HG = 1;  // kv heads per work-group (two and four side by side measured up to 8 % slower with grouped heads)
     const int phases = kRvWaves / HG;  // waves that share a kv head take the sub-tiles in turn
     const int hkRaw = blockIdx.x * HG + waveId % HG;
     const bool headLive = hkRaw < a.Hkv;
@@ -512,7 +511,6 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     int TT = 512 * a.G;
     if (TT < 2048) TT = 2048;
     if (TT > 8192) TT = 8192;
-    TT = envInt("DIOPI_ROCM_REDUCEV_TT", TT);
     TT = static_cast<int>(ceilDiv(TT, kSub)) * kSub;
     sp.TT = TT;
     sp.splits = static_cast<int>(ceilDiv(a.maxInputLen, TT));
@@ -530,9 +528,7 @@ diopiError_t launchWave(diopiContextHandle_t ctx, hipStream_t stream, void* out,
     ROCM_CHECK(sp.splits <= 65535, "max_input_len %d needs more than 65535 ranges of %d tokens", a.maxInputLen, TT);
     // kv heads per work-group: 1, 2 or 4 of the four waves' worth (the others are sub-tile phases of the same head); one
     // head per work-group measured best or equal at both shapes above (2 and 4 heads: up to 8 % slower with grouped heads)
-    int HG = envInt("DIOPI_ROCM_REDUCEV_HEADS", 1);
-    if (HG != 1 && HG != 2 && HG != 4) HG = 1;
-    sp.headsPerGroup = HG;
+    const int HG = 1;
     const dim3 grid(static_cast<unsigned>(ceilDiv(a.Hkv, HG)), static_cast<unsigned>(a.batch), static_cast<unsigned>(sp.splits));
 #define ROCM_RVW_CASE(GC)                                                                                                                   \
     hipLaunchKernelGGL((softmaxReduceVWave<T, GC>), grid, dim3(kRvThreads), 0, stream, static_cast<T*>(out), static_cast<const T*>(logits), \
@@ -584,7 +580,7 @@ diopiError_t tokenSoftmaxReduceV(diopiContextHandle_t ctx, const TensorView& vOu
     // the matrix-core kernel keeps slot numbers in 32 bits, reads V rows with 16-byte loads and addresses the G logits
     // rows of a kv head with a 32-bit byte offset
     const bool mfma = a.D == kD && a.G <= 16 && a.numSlots < (int64_t(1) << 31) && (reinterpret_cast<uintptr_t>(vV.data) & 15) == 0 &&
-                      a.logitCols * 16 * 2 < (int64_t(1) << 31) && envInt("DIOPI_ROCM_FORCE_GENERIC", 0) == 0;
+                      a.logitCols * 16 * 2 < (int64_t(1) << 31);
     switch (vOut.dtype) {
         case diopi_dtype_float16:
             return mfma ? launchWave<half_t>(ctx, stream, vOut.data, vLogits.data, vV.data, a)

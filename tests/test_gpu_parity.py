@@ -741,9 +741,58 @@ def test_decode_config3_full_size_sampled():
     assert_bit_equal(l2, logits, "relabelling the cache slots changes nothing")
 
 
+def _whole_batch_decode_checks(w, logits, out, what):
+    """Checks of a full-size decode step that cover every sequence of the batch without the CPU oracle: the logits and the
+    output against a float32 statement of the operator evaluated with torch on the device (gather, matmul, softmax, one
+    sequence at a time), the uniform-softmax closed form, and invariance under a relabelling of the cache slots."""
+    q, kc, vc = w["q"], w["k_cache"], w["v_cache"]
+    B, H, D = q.shape
+    Hkv = kc.shape[1]
+    G = H // Hkv
+    n = w["max_input_len"]
+    lens, starts = w["b_seq_len"].tolist(), w["b_start_loc"].tolist()
+    tol = TOL[q.dtype]
+    const = torch.zeros_like(logits)
+    mean_out = torch.zeros_like(out)
+    F.token_softmax_reducev(const, vc, mean_out, w["b_loc"], w["b_start_loc"], w["b_seq_len"], n, 0)
+    worst_l = worst_o = worst_m = 0.0
+    for i in range(B):
+        L, s0 = lens[i], starts[i]
+        rows = w["b_loc"][i, n - L: n].long()
+        k_rows = kc[rows].float()                                   # [L, Hkv, D]
+        qi = q[i].float().reshape(Hkv, G, D)
+        # the reference's own roundings: the dot product to the tensor dtype, then the division by sqrt(D)
+        dots = torch.einsum("hgd,lhd->hgl", qi, k_rows).to(q.dtype).float()
+        want_l = (dots / math.sqrt(D)).to(q.dtype).reshape(H, L)
+        got_l = logits[:, s0: s0 + L]
+        bad = ((got_l.float() - want_l.float()).abs() > tol["atol"] + tol["rtol"] * want_l.float().abs()).sum().item()
+        assert bad == 0, f"{what}: sequence {i} (length {L}): {bad} logits outside tolerance of the float32 statement"
+        worst_l = max(worst_l, float((got_l.float() - want_l.float()).abs().max()))
+        v_rows = vc[rows].float()
+        p = torch.softmax(got_l.float(), dim=-1).to(q.dtype).float().reshape(Hkv, G, L)
+        want_o = torch.einsum("hgl,lhd->hgd", p, v_rows).reshape(H, D)
+        assert_close(out[i], want_o, what=f"{what}: sequence {i} (length {L}) output vs the float32 statement", **tol)
+        worst_o = max(worst_o, float((out[i].float() - want_o).abs().max()))
+        want_m = v_rows.mean(0).repeat_interleave(G, dim=0)
+        assert_close(mean_out[i], want_m, what=f"{what}: sequence {i}: uniform softmax = mean of rows", **tol)
+        worst_m = max(worst_m, float((mean_out[i].float() - want_m).abs().max()))
+    say(what, "all %d sequences: max abs error logits %.3e, output %.3e, uniform %.3e" % (B, worst_l, worst_o, worst_m))
+    del const, mean_out
+    perm = torch.randperm(w["slots"], device=DEV)
+    k2 = torch.empty_like(kc)
+    k2[perm] = kc
+    l2 = torch.full_like(logits, -12288.0)
+    F.token_attention(q, k2, l2, perm[w["b_loc"].long()].int(), w["b_start_loc"], w["b_seq_len"], n)
+    assert_bit_equal(l2, logits, what + ": relabelling the cache slots changes nothing")
+
+
 def test_decode_config5_full_size_sampled():
     w = W.cfg5(DEV, seed=5)
-    _decode_case(w, torch.bfloat16, "cfg5 full, 8 sequences checked", seq_subset=[0, 17, 38, 64, 81, 99, 113, 127])
+    lens = w["b_seq_len"].tolist()
+    longest, shortest = max(range(len(lens)), key=lens.__getitem__), min(range(len(lens)), key=lens.__getitem__)
+    subset = sorted(set([0, 9, 17, 26, 38, 47, 55, 64, 72, 81, 90, 99, 106, 113, 120, 127, longest, shortest]))
+    logits, out = _decode_case(w, torch.bfloat16, f"cfg5 full, {len(subset)} sequences checked (longest and shortest among them)", seq_subset=subset)
+    _whole_batch_decode_checks(w, logits, out, "cfg5 full, whole batch")
 
 
 # ----------------------------------------------------------------------------- prefill attention
@@ -1532,6 +1581,153 @@ def test_harness_hooks_drive_an_operator_without_torch_on_the_device():
         rtl.device_free(ptr)
     assert rtl.device_destroy_stream(stream) == 0
     assert rtl.finalizeLibrary() == 0
+
+
+class _HookDevice:
+    """A caller in the manner of the reference's test runtime (litert.cpp:358-380): every device buffer comes from
+    device_malloc, every transfer is an asynchronous copy on a stream from device_make_stream, the operators are enqueued
+    on that stream through a context made for it, and the host waits with device_synchronize_stream.  No torch on the device."""
+
+    NP_DTYPES = {np.dtype(np.float16): rt.Dtype.float16, np.dtype(np.float32): rt.Dtype.float32, np.dtype(np.float64): rt.Dtype.float64,
+                 np.dtype(np.int32): rt.Dtype.int32, np.dtype(np.int64): rt.Dtype.int64}
+
+    def __init__(self):
+        import ctypes as C
+        self.C = C
+        self.rtl, self.impl = rt.libs().rt, rt.libs().impl
+        assert self.rtl.initLibrary() == 0
+        self.stream = C.c_void_p()
+        assert self.rtl.device_make_stream(C.byref(self.stream)) == 0 and self.stream.value
+        self.ctx = self.rtl.diopirtContextCreate(self.stream)
+        self.buffers, self.handles = [], []
+
+    def tensor(self, array):
+        """Device copy of a numpy array, wrapped in a tensor handle."""
+        array = np.ascontiguousarray(array)
+        ptr = self.rtl.device_malloc(max(array.nbytes, 1))
+        assert ptr
+        self.buffers.append(ptr)
+        if array.nbytes:
+            assert self.rtl.device_memcpy_h2d_async(self.stream, ptr, array.ctypes.data, array.nbytes) == 0
+            assert self.rtl.device_synchronize_stream(self.stream) == 0  # the host array may go away after this call
+        dims = (self.C.c_int64 * max(array.ndim, 1))(*array.shape)
+        h = self.rtl.diopirtTensorWrap(ptr, dims, None, array.ndim, int(self.NP_DTYPES[array.dtype]), int(rt.Device.AIChip))
+        assert h
+        self.handles.append(h)
+        return h, ptr
+
+    def fetch(self, ptr, like):
+        host = np.empty_like(like)
+        if host.nbytes:
+            assert self.rtl.device_memcpy_d2h_async(self.stream, host.ctypes.data, ptr, host.nbytes) == 0
+        assert self.rtl.device_synchronize_stream(self.stream) == 0
+        return host
+
+    def call(self, name, *args):
+        ret = getattr(self.impl, name)(self.ctx, *args)
+        assert ret == 0, f"{name}: {ret}: {rt.get_last_error_string()}"
+
+    def close(self):
+        for h in self.handles:
+            self.rtl.diopirtTensorDestroy(h)
+        self.rtl.diopirtContextDestroy(self.ctx)
+        for ptr in self.buffers:
+            self.rtl.device_free(ptr)
+        assert self.rtl.device_destroy_stream(self.stream) == 0
+        assert self.rtl.finalizeLibrary() == 0
+
+
+def test_harness_hooks_drive_the_six_hot_path_operators(golden):
+    """rms_norm, rotary_emb, destindex_copy_kv, token_attention, token_softmax_reducev and context_attention on the
+    reference's own case shapes (diopi_configs.py:9053-9105, 9137-9263, 9314-9381, 9517-9610), driven the way diopi_test
+    drives a backend: memory, copies, stream and synchronisation through the conform_test.h hooks only, results checked
+    against the oracle on the host."""
+    dev = _HookDevice()
+    rng = np.random.default_rng(17)
+    try:
+        for name in ("float32", "float16"):
+            npdt, dt = np.dtype(name), TORCH_DTYPES[name]
+            tol = TOL[dt]
+            rnd = lambda *shape: rng.standard_normal(shape).astype(npdt)  # noqa: E731
+
+            # ---- rms_norm (with the backward pass on the fp32 cases)
+            for case in golden["rms_norm"]["cases"]:
+                shape, ns, eps = case["input"], case["normalized_shape"], case["eps"]
+                x, w = rnd(*shape), rng.uniform(0.5, 1.5, ns).astype(npdt)
+                lead = shape[: len(shape) - len(ns)]
+                out, inv = np.zeros_like(x), np.zeros(lead, np.float32)
+                (hx, _), (hw, _), (ho, po), (hi, pi) = dev.tensor(x), dev.tensor(w), dev.tensor(out), dev.tensor(inv)
+                dev.call("diopiRMSNorm", ho, hi, hx, rt.Sizes(ns).c, hw, None, eps)
+                got_out, got_inv = dev.fetch(po, out), dev.fetch(pi, inv)
+                want_out, want_inv = O.rms_norm(torch.from_numpy(x), tuple(ns), torch.from_numpy(w), None, eps)
+                assert_close(torch.from_numpy(got_out), want_out, what=f"hooks: rms_norm {shape} {name}", **tol)
+                assert_close(torch.from_numpy(got_inv), want_inv, what=f"hooks: inv_rms {shape} {name}", **TOL[torch.float32])
+                if name == "float32":
+                    go = rnd(*shape)
+                    gi, gw = np.zeros_like(x), np.zeros_like(w)
+                    (hgo, _), (hgi, pgi), (hgw, pgw) = dev.tensor(go), dev.tensor(gi), dev.tensor(gw)
+                    dev.call("diopiRMSNormBackward", hgi, hgw, None, hgo, hx, hw, None, hi, rt.Sizes(ns).c, eps)
+                    want_gi, want_gw, _ = O.rms_norm_backward(torch.from_numpy(go), torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(got_inv),
+                                                              tuple(ns), exact=True)
+                    assert_close(torch.from_numpy(dev.fetch(pgi, gi)), want_gi, what=f"hooks: rms_norm grad_input {shape}", rtol=1e-5, atol=1e-5)
+                    assert_close(torch.from_numpy(dev.fetch(pgw, gw)), want_gw, what=f"hooks: rms_norm grad_weight {shape}", rtol=1e-4, atol=1e-4)
+
+            # ---- rotary_emb (the interleaved cases answer diopiNoImplement, as the reference's own implementation does)
+            for case in golden["rotary_emb"]["cases"]:
+                x, cos, sin = rnd(*case["input"]), rnd(*case["cos"]), rnd(*case["cos"])
+                out = np.zeros_like(x)
+                (hx, _), (hc, _), (hs, _), (ho, po) = dev.tensor(x), dev.tensor(cos), dev.tensor(sin), dev.tensor(out)
+                ret = dev.impl.diopiRotaryEmbedding(dev.ctx, ho, hx, hc, hs, bool(case["conj"]), bool(case["interleaved"]))
+                if case["interleaved"]:
+                    assert ret == int(rt.diopiError.diopi_no_implement)
+                    continue
+                assert ret == 0, rt.get_last_error_string()
+                want = O.rotary_emb(torch.from_numpy(x), torch.from_numpy(cos), torch.from_numpy(sin), case["conj"])
+                assert_close(torch.from_numpy(dev.fetch(po, out)), want, what=f"hooks: rotary_emb {case['input']} {name}", **tol)
+
+            # ---- destindex_copy_kv: bit for bit
+            for case in golden["destindex_copy_kv"]["cases"]:
+                k, cache = rnd(*case["k_shape"]), rnd(*case["out_shape"])
+                dest = np.asarray(case["dest_loc"], np.int32)
+                (hk, _), (hd, _), (hc, pc) = dev.tensor(k), dev.tensor(dest), dev.tensor(cache)
+                dev.call("diopiDestIndexCopyKV", hc, hk, hd)
+                want = cache.copy()
+                want[dest] = k
+                assert dev.fetch(pc, cache).tobytes() == want.tobytes(), f"hooks: destindex_copy_kv {case['k_shape']} {name}"
+
+            # ---- token_attention, then token_softmax_reducev on its logits
+            fx = golden["token_attention"]
+            q, kc, vc = rnd(*fx["q_shape"]), rnd(*fx["k_shape"]), rnd(*fx["k_shape"])
+            b_loc, b_start, b_len = (np.asarray(fx[key], np.int32) for key in ("b_loc", "b_start_loc", "b_seq_len"))
+            logits = np.full(fx["out_shape"], -7.0, npdt)
+            (hq, _), (hk, _), (hv, _), (hl, pl) = dev.tensor(q), dev.tensor(kc), dev.tensor(vc), dev.tensor(logits)
+            (hloc, _), (hst, _), (hln, _) = dev.tensor(b_loc), dev.tensor(b_start), dev.tensor(b_len)
+            dev.call("diopiTokenAttentionInference", hl, hq, hk, hloc, hst, hln, fx["max_input_len"])
+            got_l = dev.fetch(pl, logits)
+            want_l = O.token_attention(torch.from_numpy(q), torch.from_numpy(kc), torch.full(fx["out_shape"], -7.0, dtype=dt), torch.from_numpy(b_loc),
+                                       torch.from_numpy(b_start), torch.from_numpy(b_len), fx["max_input_len"])
+            assert_close(torch.from_numpy(got_l), want_l, what=f"hooks: token_attention {name}", **tol)
+            out = np.zeros(golden["token_softmax_reducev"]["out_shape"], npdt)
+            ho, po = dev.tensor(out)
+            dev.call("diopiTokenSoftmaxReduceVInference", ho, hl, hv, hloc, hst, hln, fx["max_input_len"], golden["token_softmax_reducev"]["other_kv_index"])
+            want_o = O.token_softmax_reducev(torch.from_numpy(got_l), torch.from_numpy(vc), torch.zeros(out.shape, dtype=dt), torch.from_numpy(b_loc),
+                                             torch.from_numpy(b_start), torch.from_numpy(b_len), fx["max_input_len"], 0)
+            assert_close(torch.from_numpy(dev.fetch(po, out)), want_o, what=f"hooks: token_softmax_reducev {name}", **tol)
+
+            # ---- context_attention
+            for case in golden["context_attention"]["cases"]:
+                q, k, v = (0.5 * rnd(*case["shape"]) for _ in range(3))
+                b_start, b_len = np.asarray(case["b_start_loc"], np.int32), np.asarray(case["b_seq_len"], np.int32)
+                out = np.full(case["shape"], 77.0, npdt)
+                (hq, _), (hk, _), (hv, _), (ho, po) = dev.tensor(q), dev.tensor(k), dev.tensor(v), dev.tensor(out)
+                (hst, _), (hln, _) = dev.tensor(b_start), dev.tensor(b_len)
+                dev.call("diopiContextAttentionInference", ho, hq, hk, hv, hst, hln, case["max_input_len"])
+                want = O.context_attention(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v), torch.full(case["shape"], 77.0, dtype=dt),
+                                           torch.from_numpy(b_start), torch.from_numpy(b_len), case["max_input_len"])
+                assert_close(torch.from_numpy(dev.fetch(po, out)), want, what=f"hooks: context_attention {case['shape']} {name}", **tol)
+            say("hooks:", name, "six operators on the reference's case shapes")
+    finally:
+        dev.close()
 
 
 def test_c_host_runs_operators_through_the_c_abi():
