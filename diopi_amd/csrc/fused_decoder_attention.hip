@@ -5,9 +5,9 @@
 // five lines of prose, no implementation and no test; what the prose leaves open is decided here and listed below.
 // For batch row b that is not finished, with L = sequence_lengths[b] tokens already cached:
 //   1. qkv = T(inoutput[b, :] @ qkv_weight) + qkv_bias                  [(H + 2 Hkv) * D], fp32 accumulate
-//   2. q and k heads rotate at position step - 1 - total_padding_tokens[b] with the half-split pairing of
-//      diopiRotaryEmbedding (dims j and j + D/2, angle pos * rope_theta^(-2j/D)); the sums of 1 and the rotation are
-//      done in fp32 and rounded once to the element type
+//   2. the first rot = rotary_embedding dims of q and k heads rotate at position step - 1 - total_padding_tokens[b] with the
+//      half-split pairing of diopiRotaryEmbedding (dims j and j + rot/2, angle pos * rope_theta^(-2j/rot), formed in
+//      double); the sums of 1 and the rotation are done in fp32 and rounded once to the element type
 //   3. k and v go to key_cache / value_cache [layer_id, b, kv head, L % max_seq_len, :]
 //   4. out[b, h, :] = sum_j p_j v_j over the last min(L + 1, max_seq_len) cached tokens (the new one included),
 //      p_j = exp(s_j - max s) / (sum exp(s - max s) + 1e-6), s_j = (q_h . k_j) / sqrt(D), query head h reading kv head
@@ -16,7 +16,8 @@
 // Open in the prose, fixed here: the rotary pairing (2), a circular cache window once L reaches max_seq_len (3, 4),
 // where the output lands when H*D < hidden_units (5), and that finished rows are left untouched everywhere.
 //
-// Four kernels, all on the context's stream:
+// Four kernels for 16-bit tensors with heads of 128 (three plain ones further down for everything else), all on the
+// context's stream:
 //   fusedQkvPart     the projection, HBM-bound on the weights.  Its units (a 32-row step of the hidden dimension of one
 //                    128-column head) go in equal runs to one work-group per compute unit: a compute unit draws a bounded
 //                    share of the memory bandwidth, so all of them have to pull, whatever the number of heads.  The four
@@ -65,7 +66,7 @@ struct FusedArgs {
     int B, hidden, H, Hkv, G;
     int64_t step;
     int maxSeq;
-    int rot;               // rotating dims of a head: 0 or kFD
+    int rot;               // rotating dims of a head: even, 0 .. head size
     float ropeTheta;
     int64_t layerOffset;   // elements from the start of a cache to the layer's [B, Hkv, maxSeq, D] block
 };
@@ -78,26 +79,46 @@ __device__ __forceinline__ int64_t rowLength(const FusedArgs& a, int b) {
     return L < 0 ? 0 : L;
 }
 
-// Finishes the pair (j, j + 64) of head `tile` of batch row b from the fp32 sums of the projection: rounding of the product,
-// bias, rotation, and the store to where the head belongs (q to the workspace, k and v into the cache row of the new token).
+// The rotation angle of pair j of a head at position pos: pos * theta^(-2j/rot), formed in double so that positions in the
+// hundreds of thousands keep their fraction of a turn (in fp32 the product alone is off by pos * 6e-8 radians).
+__device__ __forceinline__ void rotaryAngle(const FusedArgs& a, int b, int j, float* sn, float* cs) {
+    const int64_t pad = a.padding != nullptr ? loadIndex(a.padding, b, a.pad64) : 0;
+    const double pos = static_cast<double>(a.step - 1 - pad);
+    const double invFreq = exp2(-(2.0 * j / a.rot) * log2(static_cast<double>(a.ropeTheta)));
+    double s, c;
+    sincos(pos * invFreq, &s, &c);
+    *sn = static_cast<float>(s);
+    *cs = static_cast<float>(c);
+}
+
+// Finishes two elements of head `tile` of batch row b from the fp32 sums of the projection: rounding of the product, bias,
+// rotation, and the store to where the head belongs (q to the workspace, k and v into the cache row of the new token).
+// The 64 threads of a head: thread j < rot/2 takes the rotating pair (j, j + rot/2), the others two neighbours each of the
+// dims past `rot`, which keep their values.
 template <typename T>
 __device__ __forceinline__ void finishPair(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const T* __restrict__ bias, const FusedArgs& a,
-                                           int tile, int b, int j, float v0, float v1) {
+                                           int tile, int b, int j, const float* __restrict__ sums, int parts, int64_t partStride) {
     const bool isQ = tile < a.H;
     const bool isK = !isQ && tile < a.H + a.Hkv;
     const int head = isQ ? tile : (isK ? tile - a.H : tile - a.H - a.Hkv);
+    const int halfRot = a.rot / 2;
+    const bool pair = j < halfRot;
+    const int e0 = pair ? j : a.rot + 2 * (j - halfRot);
+    const int e1 = pair ? j + halfRot : e0 + 1;
+    float v0 = 0.f, v1 = 0.f;
+    for (int p = 0; p < parts; ++p) {
+        v0 += sums[p * partStride + e0];
+        v1 += sums[p * partStride + e1];
+    }
     // the product is rounded to the element type as a matrix product in that type would leave it
     float y0 = toFloat(fromFloat<T>(v0)), y1 = toFloat(fromFloat<T>(v1));
     if (bias != nullptr) {
-        y0 += toFloat(bias[tile * kFD + j]);
-        y1 += toFloat(bias[tile * kFD + j + kFD / 2]);
+        y0 += toFloat(bias[tile * kFD + e0]);
+        y1 += toFloat(bias[tile * kFD + e1]);
     }
-    if ((isQ || isK) && a.rot > 0) {
-        const int64_t pad = a.padding != nullptr ? loadIndex(a.padding, b, a.pad64) : 0;
-        const float pos = static_cast<float>(a.step - 1 - pad);
-        const float invFreq = exp2f(-(2.0f * static_cast<float>(j) / static_cast<float>(a.rot)) * log2f(a.ropeTheta));
+    if ((isQ || isK) && pair) {
         float sn, cs;
-        sincosf(pos * invFreq, &sn, &cs);
+        rotaryAngle(a, b, j, &sn, &cs);
         const float o0 = y0 * cs - y1 * sn;
         const float o1 = y0 * sn + y1 * cs;
         y0 = o0;
@@ -110,8 +131,8 @@ __device__ __forceinline__ void finishPair(T* __restrict__ qOut, T* __restrict__
         const int64_t slot = rowLength(a, b) % a.maxSeq;
         dst = (isK ? kCache : vCache) + a.layerOffset + ((static_cast<int64_t>(b) * a.Hkv + head) * a.maxSeq + slot) * kFD;
     }
-    dst[j] = fromFloat<T>(y0);
-    dst[j + kFD / 2] = fromFloat<T>(y1);
+    dst[e0] = fromFloat<T>(y0);
+    dst[e1] = fromFloat<T>(y1);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -264,13 +285,7 @@ __global__ __launch_bounds__(256) void fusedQkvFinish(T* __restrict__ qOut, T* _
         const int b = blockIdx.y * 4 + idx / (kFD / 2);
         const int j = idx % (kFD / 2);
         if (b >= a.B || rowFinished(a, b)) continue;
-        float v0 = 0.f, v1 = 0.f;
-        for (int p = 0; p < parts; ++p) {
-            const float* src = hiddenPart + (static_cast<int64_t>(p) * a.B + b) * N + tile * kFD;
-            v0 += src[j];
-            v1 += src[j + kFD / 2];
-        }
-        finishPair<T>(qOut, kCache, vCache, bias, a, tile, b, j, v0, v1);
+        finishPair<T>(qOut, kCache, vCache, bias, a, tile, b, j, hiddenPart + static_cast<int64_t>(b) * N + tile * kFD, parts, static_cast<int64_t>(a.B) * N);
     }
 }
 
@@ -543,6 +558,154 @@ __global__ __launch_bounds__(256) void fusedDecodeMerge(T* __restrict__ out, Fus
     out[static_cast<int64_t>(b) * a.hidden + idx] = static_cast<T>(num / (den + 1e-6f));
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The plain path: any of float32 / float16 / bfloat16, heads of up to kPlainMaxD dims, any even number of rotating dims, any
+// grouping of query heads and any hidden size or alignment.  Three kernels with scalar accesses and fp32 arithmetic, the
+// same five steps as above; what the fast path cannot take comes here, at a fraction of its speed.
+constexpr int kPlainMaxD = 512;
+constexpr int kPlainCols = 64;   // columns of the projection per work-group (one per lane of a wave)
+constexpr int kPlainRows = 8;    // batch rows per work-group of the projection
+constexpr int kPlainSplit = 4;   // waves of a work-group, each with every fourth row of the weights
+
+// staged[b, c] = float(T(inoutput[b, :] . qkv_weight[:, c])) + bias[c]
+template <typename T>
+__global__ __launch_bounds__(kPlainCols * kPlainSplit) void plainQkv(float* __restrict__ staged, const T* __restrict__ x, const T* __restrict__ w,
+                                                                    const T* __restrict__ bias, FusedArgs a, int N) {
+    __shared__ float part[kPlainSplit][kPlainRows][kPlainCols];
+    const int lane = threadIdx.x % kPlainCols, wave = threadIdx.x / kPlainCols;
+    const int c = blockIdx.x * kPlainCols + lane;
+    const int b0 = blockIdx.y * kPlainRows;
+    const int rows = min(kPlainRows, a.B - b0);
+    float acc[kPlainRows];
+#pragma unroll
+    for (int r = 0; r < kPlainRows; ++r) acc[r] = 0.f;
+    if (c < N) {
+        for (int h = wave; h < a.hidden; h += kPlainSplit) {
+            const float wv = toFloat(w[static_cast<int64_t>(h) * N + c]);
+#pragma unroll
+            for (int r = 0; r < kPlainRows; ++r) {
+                if (r < rows) acc[r] = fmaf(toFloat(x[static_cast<int64_t>(b0 + r) * a.hidden + h]), wv, acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kPlainRows; ++r) part[wave][r][lane] = acc[r];
+    __syncthreads();
+    for (int r = wave; r < rows; r += kPlainSplit) {
+        if (c >= N) continue;
+        float sum = 0.f;
+#pragma unroll
+        for (int p = 0; p < kPlainSplit; ++p) sum += part[p][r][lane];
+        float y = toFloat(fromFloat<T>(sum));
+        if (bias != nullptr) y += toFloat(bias[c]);
+        staged[static_cast<int64_t>(b0 + r) * N + c] = y;
+    }
+}
+
+// Rotation and placement of one head of one batch row: q to the workspace, k and v into the cache row of the new token.
+template <typename T>
+__global__ __launch_bounds__(128) void plainFinish(T* __restrict__ qOut, T* __restrict__ kCache, T* __restrict__ vCache, const float* __restrict__ staged,
+                                                  FusedArgs a, int D) {
+    const int tile = blockIdx.x, b = blockIdx.y;
+    if (rowFinished(a, b)) return;
+    const bool isQ = tile < a.H;
+    const bool isK = !isQ && tile < a.H + a.Hkv;
+    const int head = isQ ? tile : (isK ? tile - a.H : tile - a.H - a.Hkv);
+    const float* src = staged + (static_cast<int64_t>(b) * (a.H + 2 * a.Hkv) + tile) * D;
+    T* dst;
+    if (isQ) {
+        dst = qOut + (static_cast<int64_t>(b) * a.H + head) * D;
+    } else {
+        const int64_t slot = rowLength(a, b) % a.maxSeq;
+        dst = (isK ? kCache : vCache) + a.layerOffset + ((static_cast<int64_t>(b) * a.Hkv + head) * a.maxSeq + slot) * D;
+    }
+    const int halfRot = a.rot / 2;
+    for (int j = threadIdx.x; j < D; j += blockDim.x) {
+        float y = src[j];
+        if ((isQ || isK) && j < a.rot) {
+            const bool low = j < halfRot;
+            float sn, cs;
+            rotaryAngle(a, b, low ? j : j - halfRot, &sn, &cs);
+            y = low ? y * cs - src[j + halfRot] * sn : src[j - halfRot] * sn + y * cs;
+        }
+        dst[j] = fromFloat<T>(y);
+    }
+}
+
+// One wave per (query head, batch row): the lanes split the head's dims, the cached tokens of the window go by one at a
+// time with a running maximum and denominator (fp32).
+template <typename T>
+__global__ __launch_bounds__(kWave) void plainDecodeAttn(T* __restrict__ out, const T* __restrict__ qIn, const T* __restrict__ kCache, const T* __restrict__ vCache,
+                                                        FusedArgs a, int D) {
+    constexpr int kPer = kPlainMaxD / kWave;
+    const int h = blockIdx.x, b = blockIdx.y;
+    if (rowFinished(a, b)) return;
+    const int lane = threadIdx.x;
+    const int64_t L = rowLength(a, b);
+    const int64_t n = L + 1 < a.maxSeq ? L + 1 : a.maxSeq;
+    const int64_t headOff = a.layerOffset + (static_cast<int64_t>(b) * a.Hkv + h / a.G) * a.maxSeq * D;
+    const T* q = qIn + (static_cast<int64_t>(b) * a.H + h) * D;
+    const float scale = 1.0f / sqrtf(static_cast<float>(D));
+    float qv[kPer], acc[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        const int d = lane + kWave * i;
+        qv[i] = d < D ? toFloat(q[d]) : 0.f;
+        acc[i] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t row = (L + 1 - n + t) % a.maxSeq;
+        const T* kr = kCache + headOff + row * D;
+        const T* vr = vCache + headOff + row * D;
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int d = lane + kWave * i;
+            if (d < D) dot = fmaf(qv[i], toFloat(kr[d]), dot);
+        }
+        // the score as token attention leaves it: the dot product and its scaling each rounded to the element type
+        const float sc = toFloat(fromFloat<T>(toFloat(fromFloat<T>(waveSum(dot))) * scale));
+        const float mNew = fmaxf(m, sc);
+        const float corr = expf(m - mNew);  // 0 at the first token
+        const float p = expf(sc - mNew);
+        l = l * corr + p;
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int d = lane + kWave * i;
+            if (d < D) acc[i] = fmaf(p, toFloat(vr[d]), acc[i] * corr);
+        }
+        m = mNew;
+    }
+    const float inv = 1.0f / (l + 1e-6f);
+    T* o = out + static_cast<int64_t>(b) * a.hidden + static_cast<int64_t>(h) * D;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        const int d = lane + kWave * i;
+        if (d < D) o[d] = fromFloat<T>(acc[i] * inv);
+    }
+}
+
+template <typename T>
+diopiError_t launchPlain(hipStream_t stream, void* inout, const void* w, const void* bias, void* workspace, void* kCache, void* vCache, const FusedArgs& a, int D,
+                         int64_t qBytes) {
+    T* qBuf = static_cast<T*>(workspace);
+    float* staged = reinterpret_cast<float*>(static_cast<char*>(workspace) + qBytes);
+    const int tiles = a.H + 2 * a.Hkv;
+    const int N = tiles * D;
+    const dim3 pgrid(static_cast<unsigned>(ceilDiv(N, kPlainCols)), static_cast<unsigned>(ceilDiv(a.B, kPlainRows)));
+    hipLaunchKernelGGL((plainQkv<T>), pgrid, dim3(kPlainCols * kPlainSplit), 0, stream, staged, static_cast<const T*>(inout), static_cast<const T*>(w),
+                       static_cast<const T*>(bias), a, N);
+    ROCM_LAUNCH_CHECK();
+    hipLaunchKernelGGL((plainFinish<T>), dim3(static_cast<unsigned>(tiles), static_cast<unsigned>(a.B)), dim3(128), 0, stream, qBuf, static_cast<T*>(kCache),
+                       static_cast<T*>(vCache), staged, a, D);
+    ROCM_LAUNCH_CHECK();
+    hipLaunchKernelGGL((plainDecodeAttn<T>), dim3(static_cast<unsigned>(a.H), static_cast<unsigned>(a.B)), dim3(kWave), 0, stream, static_cast<T*>(inout), qBuf,
+                       static_cast<const T*>(kCache), static_cast<const T*>(vCache), a, D);
+    ROCM_LAUNCH_CHECK();
+    return diopiSuccess;
+}
+
 template <typename T>
 diopiError_t launchFused(hipStream_t stream, void* inout, const void* w, const void* bias, void* workspace, void* kCache, void* vCache, const FusedArgs& a,
                          const AttnSplit& spIn, int64_t qBytes, const ProjPlan& pl) {
@@ -606,8 +769,9 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     ROCM_CHECK(H * D <= hidden, "the attention output [local_head_num * size_per_head = %lld] does not fit hidden_units = %lld", static_cast<long long>(H * D),
                static_cast<long long>(hidden));
     ROCM_CHECK(max_seq_len > 0 && max_seq_len < (int64_t(1) << 31) / D, "max_seq_len %lld is out of range", static_cast<long long>(max_seq_len));
-    ROCM_CHECK(vK.ndim == 5 && vK.shape[1] == B && vK.shape[2] == Hkv && vK.shape[3] == max_seq_len && vK.shape[4] == D && vK.dtype == vX.dtype,
-               "key_cache must be [num_layer, batch, local_kv_head_num, max_seq_len, size_per_head] of dtype %s", dtypeName(vX.dtype));
+    // the caches may be allocated for more rows than this call's batch: the layer stride comes from their own batch dimension
+    ROCM_CHECK(vK.ndim == 5 && vK.shape[1] >= B && vK.shape[2] == Hkv && vK.shape[3] == max_seq_len && vK.shape[4] == D && vK.dtype == vX.dtype,
+               "key_cache must be [num_layer, batch >= batch_size, local_kv_head_num, max_seq_len, size_per_head] of dtype %s", dtypeName(vX.dtype));
     ROCM_CHECK(vV.sameShape(vK) && vV.dtype == vK.dtype, "value_cache must have the shape and dtype of key_cache");
     ROCM_CHECK(layer_id >= 0 && layer_id < vK.shape[0], "layer_id %lld is outside the %lld layers of the caches", static_cast<long long>(layer_id),
                static_cast<long long>(vK.shape[0]));
@@ -636,19 +800,17 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
         a.padding = vP.data;
         a.pad64 = vP.dtype == diopi_dtype_int64;
     }
-    // what this build implements: 16-bit elements, heads of 128, up to 16 query heads per kv head, rotation of the whole head
-    // or none, a hidden size in whole 32-row steps for each of a work-group's four waves, 16-byte aligned rows
-    const bool supported = (vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16) && D == kFD && H / Hkv <= 16 &&
-                           (rotary_embedding == 0 || rotary_embedding == kFD) && hidden % 128 == 0 && hidden >= 256 &&
-                           ((reinterpret_cast<uintptr_t>(vX.data) | reinterpret_cast<uintptr_t>(vW.data) | reinterpret_cast<uintptr_t>(vK.data) |
-                             reinterpret_cast<uintptr_t>(vV.data)) & 15) == 0;
-    if (!supported) {
-        setLastError("diopiFusedDecoderAttentionInp: only float16 / bfloat16, size_per_head 128, at most 16 query heads per kv head, rotary_embedding 0 or "
-                     "128 and hidden_units a multiple of 128 are implemented (got %s, %lld, %lld, %lld, %lld)",
-                     dtypeName(vX.dtype), static_cast<long long>(D), static_cast<long long>(H / Hkv), static_cast<long long>(rotary_embedding),
-                     static_cast<long long>(hidden));
-        return diopiNoImplement;
-    }
+    ROCM_CHECK(vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16 || vX.dtype == diopi_dtype_float32,
+               "inoutput must be float16, bfloat16 or float32, got %s", dtypeName(vX.dtype));
+    ROCM_CHECK(D > 0 && D <= kPlainMaxD, "size_per_head %lld is outside 1..%d", static_cast<long long>(D), kPlainMaxD);
+    ROCM_CHECK(rotary_embedding >= 0 && rotary_embedding <= D && rotary_embedding % 2 == 0, "rotary_embedding %lld must be even and within 0..size_per_head = %lld",
+               static_cast<long long>(rotary_embedding), static_cast<long long>(D));
+    ROCM_CHECK(B <= 65535 && H <= 65535, "batch %lld / local_head_num %lld exceed the launch limits", static_cast<long long>(B), static_cast<long long>(H));
+    // the fast path: 16-bit elements, heads of 128, up to 16 query heads per kv head, a hidden size in whole 32-row steps for
+    // each of a work-group's four waves, 16-byte aligned rows; everything else goes to the plain kernels
+    const bool fast = (vX.dtype == diopi_dtype_float16 || vX.dtype == diopi_dtype_bfloat16) && D == kFD && H / Hkv <= 16 && hidden % 128 == 0 && hidden >= 256 &&
+                      ((reinterpret_cast<uintptr_t>(vX.data) | reinterpret_cast<uintptr_t>(vW.data) | reinterpret_cast<uintptr_t>(vK.data) |
+                        reinterpret_cast<uintptr_t>(vV.data)) & 15) == 0;
     // ranges of the attention kernel: 1024 cached tokens per work-group (its four waves share them), the workspace sized for
     // max_seq_len.  Measured at 64 rows of 512..2047 tokens, 32 kv heads, items taken longest first: 1024 tokens per range
     // 237-238 us per call in two harnesses, 512: 247-251, 2048 (no partials, no merge launch): 235 in one, 254 in the other
@@ -658,8 +820,7 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     sp.splits = static_cast<int>(ceilDiv(max_seq_len, sp.TT));
     sp.partAcc = nullptr;
     sp.partMl = nullptr;
-    ROCM_CHECK(B <= 65535 && sp.splits <= 65535, "batch %lld / max_seq_len %lld exceed the launch limits", static_cast<long long>(B),
-               static_cast<long long>(max_seq_len));
+    ROCM_CHECK(sp.splits <= 65535, "max_seq_len %lld exceeds the launch limits", static_cast<long long>(max_seq_len));
     const int64_t e = vX.itemsize();
     const int64_t qBytes = ceilDiv(B * H * D * e, 256) * 256;
     const int64_t attnBytes = sp.splits > 1 ? B * sp.splits * H * (D + 2) * static_cast<int64_t>(sizeof(float)) : 0;
@@ -668,7 +829,9 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     ProjPlan pl;
     pl.tiles = static_cast<int>(H + 2 * Hkv);
     pl.stepsPerTile = static_cast<int>(hidden / 32);
-    {
+    pl.unitsPerWg = 1;
+    pl.slots = 1;
+    if (fast) {
         const int64_t units = static_cast<int64_t>(pl.tiles) * pl.stepsPerTile;
         const int64_t rowBlocks = ceilDiv(B > 0 ? B : 1, kProjRows);
         // when the heads are fewer than the compute units a head is cut into as many equal runs as fit (runs that end with
@@ -683,7 +846,8 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
         for (int t = 0; t < pl.tiles; ++t) pl.slots = std::max(pl.slots, projLastWg(pl, t) - projFirstWg(pl, t) + 1);
     }
     const int64_t projBytes = static_cast<int64_t>(pl.slots) * B * N * static_cast<int64_t>(sizeof(float));
-    const int64_t need = qBytes + (attnBytes > projBytes ? attnBytes : projBytes);
+    const int64_t stagedBytes = B * N * static_cast<int64_t>(sizeof(float));  // the plain path's projection, fp32
+    const int64_t need = qBytes + (fast ? (attnBytes > projBytes ? attnBytes : projBytes) : stagedBytes);
     if (*workspace_size < 0) {
         *workspace_size = need;  // size query: nothing else happens
         return diopiSuccess;
@@ -711,9 +875,15 @@ diopiError_t fusedDecoderAttention(diopiContextHandle_t ctx, diopiTensorHandle_t
     a.maxSeq = static_cast<int>(max_seq_len);
     a.rot = static_cast<int>(rotary_embedding);
     a.ropeTheta = rope_theta;
-    a.layerOffset = layer_id * B * Hkv * max_seq_len * D;
+    a.layerOffset = layer_id * vK.shape[1] * Hkv * max_seq_len * D;
     hipStream_t stream;
     ROCM_CALL(getStream(ctx, &stream));
+    if (!fast) {
+        const int d = static_cast<int>(D);
+        if (vX.dtype == diopi_dtype_float32) return launchPlain<float>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, d, qBytes);
+        if (vX.dtype == diopi_dtype_float16) return launchPlain<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, d, qBytes);
+        return launchPlain<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, d, qBytes);
+    }
     if (vX.dtype == diopi_dtype_float16) return launchFused<half_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, pl);
     return launchFused<bf16_t>(stream, vX.data, vW.data, biasPtr, wsPtr, vK.data, vV.data, a, sp, qBytes, pl);
 }

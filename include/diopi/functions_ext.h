@@ -148,7 +148,9 @@ DIOPI_API diopiError_t diopiContextAttentionInference(diopiContextHandle_t ctx, 
  * the query tiles is kept in a static device array of the library (128 KiB per device, held until the process ends).
  * Limit: ceil(rows / BM) + batch <= 8192 (BM = 256 query rows once the sequences average 1024 rows or more, else
  * 128); a larger call returns diopiErrorOccurred with a message.  All calls on one device share the array: calls that
- * overlap on one device (different streams or threads) race on it and must be serialised by the caller.
+ * overlap on one device (different streams or threads) race on it and must be serialised by the caller.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress) and reads the device's properties, neither of
+ * which may be recorded into a graph: make one ordinary call on each device before the first capture.
  */
 DIOPI_API diopiError_t diopiContextAttentionInferenceNoAlloc(diopiContextHandle_t ctx, diopiTensorHandle_t context_attention_out, diopiConstTensorHandle_t q,
                                                              diopiConstTensorHandle_t k, diopiConstTensorHandle_t v, diopiConstTensorHandle_t b_start_loc,

@@ -42,21 +42,25 @@ DIOPI_API diopiError_t diopiFusedAddRootMeanSquareNormInp(diopiContextHandle_t c
  * One decode step of self-attention behind a single call (reference: functions_lmdeploy.h:104-135): QKV projection,
  * bias, rotary embedding, insertion of the new key/value rows into the caches, and attention of the new token over its
  * sequence's cached tokens, without any intermediate tensor in HBM but the projected query.
- *   inoutput   [batch_size, hidden_units] float16 / bfloat16; in: hidden states, out: columns 0 .. H*D-1 hold the
+ *   inoutput   [batch_size, hidden_units] float16 / bfloat16 / float32; in: hidden states, out: columns 0 .. H*D-1 hold the
  *              attention output of every row that is not finished (H*D <= hidden_units)
  *   qkv_weight [hidden_units, (H + 2 Hkv) * D], qkv_bias [(H + 2 Hkv) * D] or a null handle: query heads, then key
  *              heads, then value heads along the second axis
  *   workspace / workspace_size: *workspace_size < 0 only writes the bytes the call needs into *workspace_size; else
  *              `workspace` (any dtype, 16-byte aligned) must hold that many bytes.  A null workspace handle with a
  *              non-negative size takes the bytes from the context (diopiRequireBuffer)
- *   key_cache, value_cache [num_layer, batch_size, Hkv, max_seq_len, D]: row sequence_lengths[b] % max_seq_len of layer
- *              layer_id receives the new key / value of row b
+ *   key_cache, value_cache [num_layer, rows >= batch_size, Hkv, max_seq_len, D]: row sequence_lengths[b] % max_seq_len of
+ *              layer layer_id receives the new key / value of row b
  *   finished [batch_size] bool or null; total_padding_tokens [batch_size] int32/int64 or null (zeros);
  *   sequence_lengths [batch_size] int32/int64: tokens already cached; step: the rotary position is
- *              step - 1 - total_padding_tokens[b]; rotary_embedding: rotating dims of a head (0 or D); rope_theta: base
+ *              step - 1 - total_padding_tokens[b]; rotary_embedding: rotating dims of a head (even, 0 .. D: the
+ *              first rotary_embedding dims pair up as j and j + rotary_embedding/2, the rest keep their values); rope_theta: base
  * Attention runs over the last min(sequence_lengths[b] + 1, max_seq_len) tokens, scores scaled by 1/sqrt(D), softmax
- * denominator + 1e-6.  Implemented for D = 128 and H / Hkv <= 16 (else diopiNoImplement).  fusion_level is accepted
- * and ignored.  HBM-bound: the weight matrix once, then one K row and one V row per cached token.
+ * denominator + 1e-6.  fusion_level is accepted and ignored.  Two sets of kernels: float16 / bfloat16 with D = 128,
+ * H / Hkv <= 16, hidden_units a multiple of 128 and 16-byte aligned tensors run on the matrix cores, HBM-bound (the weight
+ * matrix once, then one K row and one V row per cached token); every other combination (float32, D up to 512, any grouping,
+ * size or alignment) runs plain kernels with the same results at a fraction of that speed.  An odd rotary_embedding,
+ * D > 512 or another dtype is an error (diopiErrorOccurred).
  */
 DIOPI_API diopiError_t diopiFusedDecoderAttentionInp(diopiContextHandle_t ctx, diopiTensorHandle_t inoutput, diopiConstTensorHandle_t qkv_weight,
                                                      diopiConstTensorHandle_t qkv_bias, diopiTensorHandle_t workspace, int64_t* workspace_size,

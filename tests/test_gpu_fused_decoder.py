@@ -1,6 +1,7 @@
 """Parity of diopiFusedDecoderAttentionInp (called through the C ABI) against the CPU oracle's composition of the
-reference's pinned parts.  Bar: 16-bit tensors within atol = rtol = 1e-2 of the dtype-faithful composition and of float64;
-the cache rows the call writes are compared the same way, every other cache row bit for bit."""
+reference's pinned parts.  Bar: 16-bit tensors within atol = rtol = 1e-2, float32 tensors within atol = rtol = 1e-5, of the
+dtype-faithful composition and of float64; the cache rows the call writes are compared the same way, every other cache row
+bit for bit."""
 import ctypes
 import math
 
@@ -21,28 +22,39 @@ def say(*a):
 
 
 def _case(B, H, Hkv, S, seq, dt, seed, hidden=None, layers=2, layer=1, pad=None, finished=None, step=None, bias=True, rot=128, idt=torch.int32,
-          theta=10000.0, what="", out_mismatch=0.0):
-    D = 128
+          theta=10000.0, what="", out_mismatch=0.0, D=128, cache_rows=None, misalign=False):
+    """cache_rows: batch dimension of the caches when larger than B (rows past B must stay untouched); misalign: every
+    tensor starts one element past a 16-byte boundary."""
     g = torch.Generator().manual_seed(seed)
     hid = H * D if hidden is None else hidden
     N = (H + 2 * Hkv) * D
     x = torch.randn(B, hid, generator=g).to(dt)
     w = (torch.randn(hid, N, generator=g) / math.sqrt(hid)).to(dt)
     b = torch.randn(N, generator=g).to(dt) if bias else None
-    kc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dt)
-    vc = torch.randn(layers, B, Hkv, S, D, generator=g).to(dt)
+    CB = B if cache_rows is None else cache_rows
+    kc = torch.randn(layers, CB, Hkv, S, D, generator=g).to(dt)
+    vc = torch.randn(layers, CB, Hkv, S, D, generator=g).to(dt)
     seq_t = torch.tensor(seq, dtype=idt)
     pad_t = None if pad is None else torch.tensor(pad, dtype=idt)
     fin_t = None if finished is None else torch.tensor(finished, dtype=torch.bool)
     step = max(seq) + 1 if step is None else step
-    say("fused decoder attention", what, dict(B=B, H=H, Hkv=Hkv, S=S, hidden=hid, dtype=str(dt), seq=seq[:8], step=step))
+    say("fused decoder attention", what, dict(B=B, H=H, Hkv=Hkv, D=D, S=S, hidden=hid, rot=rot, dtype=str(dt), seq=seq[:8], step=step))
     # oracle, dtype-faithful and float64 (each on its own copy of the caches)
     rk, rv = kc.clone(), vc.clone()
     ref = O.fused_decoder_attention_inp(x, w, b, rk, rv, fin_t, pad_t, seq_t, step, layer, H, Hkv, D, S, rot, theta)
     ek, ev = kc.double(), vc.double()
     ex = O.fused_decoder_attention_inp(x, w, b, ek, ev, fin_t, pad_t, seq_t, step, layer, H, Hkv, D, S, rot, theta, exact=True)
     # device
-    xd, wd, bd, kd, vd = x.to(DEV), w.to(DEV), (None if b is None else b.to(DEV)), kc.to(DEV), vc.to(DEV)
+    def put(t):
+        if t is None or not misalign:
+            return None if t is None else t.to(DEV)
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=DEV)
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 != 0
+        return view
+
+    xd, wd, bd, kd, vd = put(x), put(w), put(b), put(kc), put(vc)
     args = [t if t is None else t.to(DEV) for t in (fin_t, pad_t, seq_t)]
     w_before = wd.clone()
     out = F.fused_decoder_attention_inp(xd, wd, bd, None, 0, kd, vd, args[0], args[1], args[2], step, layer, H, Hkv, D, S, rot, theta)
@@ -52,7 +64,7 @@ def _case(B, H, Hkv, S, seq, dt, seed, hidden=None, layers=2, layer=1, pad=None,
     assert_close(out, ex, what=what + " output vs float64", mismatch_ratio=out_mismatch, **tol)
     say(what, "max_abs/rel vs f64: %.3e %.3e" % report(out, ex))
     # caches: the written rows within tolerance, every other row untouched
-    written = torch.zeros(layers, B, Hkv, S, dtype=torch.bool)
+    written = torch.zeros(layers, CB, Hkv, S, dtype=torch.bool)
     for i in range(B):
         if finished is None or not finished[i]:
             written[layer, i, :, seq[i] % S] = True
@@ -162,12 +174,53 @@ def test_fused_decoder_attention_workspace_protocol_and_errors():
     ctx.clear_tensors()
     assert_bit_equal(x1, x2, "workspace tensor vs context scratch")
     assert_bit_equal(k1, k2, "workspace tensor vs context scratch: key cache")
-    # shapes this build does not implement answer diopiNoImplement (13)
-    x64 = torch.randn(B, 4 * 64, dtype=torch.float16, device=DEV)
-    w64 = torch.randn(4 * 64, 3 * 4 * 64, dtype=torch.float16, device=DEV)
-    k64 = torch.zeros(1, B, 4, S, 64, dtype=torch.float16, device=DEV)
+    # an odd number of rotating dims is refused with a message
+    r = impl.diopiFusedDecoderAttentionInp(ctx.handle, hx.handle, hw.handle, None, None, ctypes.byref(ctypes.c_int64(-1)), *(tail[:-2] + (33, 10000.0)))
+    assert r != 0 and b"rotary_embedding" in impl.diopiGetLastErrorString()
+    # float64 tensors are refused
+    x64, w64, k64 = x.double(), w.double(), kc.double()
     v64 = k64.clone()
     hx64, hw64, hk64, hv64 = (rt.Tensor(t) for t in (x64, w64, k64, v64))
     r = impl.diopiFusedDecoderAttentionInp(ctx.handle, hx64.handle, hw64.handle, None, None, ctypes.byref(ctypes.c_int64(-1)), 0, hk64.handle, hv64.handle,
-                                           None, None, hs.handle, 10, 0, 4, 4, 64, S, 64, 10000.0)
-    assert r == 13, r
+                                           *tail[3:])
+    assert r != 0 and b"float16, bfloat16 or float32" in impl.diopiGetLastErrorString()
+
+
+def test_fused_decoder_attention_partial_rotation_on_heads_of_128():
+    # the first 64 (32, 2) dims of a head rotate, the rest keep their values
+    for dt, rot, seed in ((torch.float16, 64, 21), (torch.bfloat16, 32, 22), (torch.float16, 2, 23)):
+        _case(B=5, H=4, Hkv=2, S=300, seq=[0, 17, 299, 150, 64], dt=dt, seed=seed, rot=rot, pad=[0, 1, 2, 3, 4], step=310, what=f"rotary {rot} of 128")
+
+
+def test_fused_decoder_attention_float32_and_other_head_sizes():
+    """What the fast kernels do not take goes through the plain kernels: float32 tensors, heads of 64 / 80 / 256 dims, partial
+    rotation there, more than 16 query heads per kv head, a hidden size that is no multiple of 128, unaligned tensors."""
+    _case(B=5, H=4, Hkv=4, S=64, seq=[0, 1, 31, 40, 63], dt=torch.float32, seed=31, what="float32 MHA")
+    _case(B=9, H=6, Hkv=2, S=50, seq=[0, 49, 120, 7, 50, 51, 99, 100, 3], dt=torch.float32, seed=32, D=64, rot=32, pad=[0, 1, 0, 2, 0, 3, 0, 4, 0],
+          finished=[False] * 8 + [True], step=130, idt=torch.int64, what="float32 heads of 64, rotary 32, wrap")
+    _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float16, seed=33, D=80, rot=40, hidden=4 * 80 + 8, what="fp16 heads of 80, rotary 40")
+    _case(B=2, H=2, Hkv=1, S=33, seq=[32, 8], dt=torch.bfloat16, seed=34, D=256, rot=256, bias=False, what="bf16 heads of 256")
+    _case(B=4, H=32, Hkv=1, S=70, seq=[69, 0, 33, 12], dt=torch.float16, seed=35, what="32 query heads on one kv head")
+    _case(B=3, H=1, Hkv=1, S=20, seq=[19, 3, 10], dt=torch.float16, seed=36, hidden=200, what="hidden 200")
+    _case(B=3, H=2, Hkv=2, S=20, seq=[19, 3, 10], dt=torch.float16, seed=37, misalign=True, what="unaligned tensors")
+    _case(B=3, H=2, Hkv=2, S=20, seq=[19, 3, 10], dt=torch.float32, seed=38, rot=0, layers=3, layer=2, what="float32 no rotation, layer 2")
+
+
+def test_fused_decoder_attention_caches_with_more_rows_than_the_batch():
+    # the layer stride follows the caches' own batch dimension; rows past the batch stay as they are
+    _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float16, seed=41, cache_rows=7, layers=3, layer=2, what="cache of 7 rows, fast path")
+    _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float32, seed=42, cache_rows=5, layers=2, layer=1, D=64, rot=64, what="cache of 5 rows, plain path")
+
+
+def test_fused_decoder_attention_far_positions():
+    # position 100000: the angle needs more than fp32 (100000 * 6e-8 = 6e-3 radians of error otherwise)
+    _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float16, seed=51, pad=[0, 7, 50000], step=100001, what="position 1e5, fast path")
+    _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float32, seed=52, pad=[0, 7, 50000], step=100001, D=64, rot=64, what="position 1e5, float32")
+
+
+def test_fused_decoder_attention_more_items_than_the_ranking_takes():
+    # 200 rows x 2 ranges of 1024 tokens are 400 items per kv head: past the 256 that are taken longest first, the plain order
+    g = torch.Generator().manual_seed(61)
+    seq = torch.randint(0, 2048, (200,), generator=g).tolist()
+    seq[0], seq[1], seq[2] = 2047, 0, 1024
+    _case(B=200, H=2, Hkv=1, S=2048, seq=seq, dt=torch.float16, seed=61, layers=1, layer=0, hidden=256, what="200 rows, 2 ranges")
