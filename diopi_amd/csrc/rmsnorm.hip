@@ -259,7 +259,7 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 
 // ---------------------------------------------------------------------------
 // Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
-// A work-group is GROUPS row teams of 256 threads.  In step i, team g of work-group b takes row
+// A work-group is GROUPS row teams of 256 threads, WGS of them resident on a compute unit.  In step i, team g of work-group b takes row
 // (i * gridDim.x + b) * GROUPS + g: at any moment the whole grid works on one contiguous window of
 // gridDim.x * GROUPS rows of each tensor, which spreads the traffic evenly over the memory channels (a private run of
 // rows per work-group would put the work-groups, which advance in step, a fixed large stride apart).
@@ -275,9 +275,13 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 //
 // The column sums for grad_weight / grad_bias are accumulated in fp32 registers and moved every kBwdFlush steps into
 // per-team LDS arrays of ColAcc (fp64 for fp32 tensors), which bounds the length of any fp32 summation; at the end
-// the team arrays are summed in a fixed order into one partial row per work-group.  One large work-group per compute
-// unit keeps the partial buffer at one row per unit.  The row sum s[r] crosses the team's four waves through LDS:
-// one barrier per step.
+// the team arrays are summed in a fixed order into one fp32 partial row per work-group (one rounding of a sum that the
+// fold then continues in fp64: the error stays below one rounding of the fp32 result).  Without grad_bias a compute
+// unit holds two work-groups of two teams: the same 16 waves and 128 KiB of LDS as one work-group of four teams, but
+// the row stream runs 5 % faster that way (6.07 against 5.79 TB/s at fp32 [8192, 4096] with the partial rows and the
+// fold taken out of both builds; the barrier is not the reason, a build without it runs at the same speed), which pays
+// for the second partial row per unit once the partial rows are fp32.  The row sum s[r] crosses the team's four waves
+// through LDS: one barrier per step.
 // ---------------------------------------------------------------------------
 constexpr int kBwdTeam = 256;
 constexpr int kBwdTeamWaves = kBwdTeam / kWave;
@@ -290,8 +294,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rowBuffer(const T* base, int64
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base + row * n2), 0, valid ? n2 * static_cast<int>(sizeof(T)) : 0, kBufferWord3);
 }
 
-template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS>
-__global__ __launch_bounds__(kBwdTeam* GROUPS) void rmsNormBwdFused(T* __restrict__ gradInput, ColAcc* __restrict__ partW, ColAcc* __restrict__ partB,
+// WGS work-groups of GROUPS teams share a compute unit: GROUPS * WGS waves on each of its four SIMDs, which is what the
+// second launch bound states (and what sets the registers a lane may use).
+template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS, int WGS>
+__global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused(T* __restrict__ gradInput, float* __restrict__ partW, float* __restrict__ partB,
                                                                        const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
                                                                        const float* __restrict__ invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
@@ -436,55 +442,61 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS) void rmsNormBwdFused(T* __restric
                 sw += sAcc[g * kCols + idx];
                 if (HAS_GBIAS) sb += sAcc[(GROUPS + g) * kCols + idx];
             }
-            partW[static_cast<int64_t>(blockIdx.x) * n2 + col] = sw;
-            if (HAS_GBIAS) partB[static_cast<int64_t>(blockIdx.x) * n2 + col] = sb;
+            partW[static_cast<int64_t>(blockIdx.x) * n2 + col] = static_cast<float>(sw);
+            if (HAS_GBIAS) partB[static_cast<int64_t>(blockIdx.x) * n2 + col] = static_cast<float>(sb);
         }
     }
 }
 
-// Folds the [numParts, n2] partial sums into grad_weight (and grad_bias) in fp64.  A 256-thread group covers
-// kCols = 128 bytes of consecutive columns x (256 / kCols) slices of the partial rows, so that n2 = 4096 spreads over
-// 128 (fp32 partials) or 256 (fp64 partials) work-groups.
-template <typename T, typename ColAcc>
-__global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight, T* __restrict__ gradBias, const ColAcc* __restrict__ partW,
-                                                       const ColAcc* __restrict__ partB, int numParts, int n2) {
-    constexpr int kCols = 128 / static_cast<int>(sizeof(ColAcc));
-    constexpr int kSlices = 256 / kCols;
-    __shared__ double red[2][kSlices][kCols];
-    const int c = threadIdx.x % kCols;
-    const int slice = threadIdx.x / kCols;
-    const int col = blockIdx.x * kCols + c;
-    double sw = 0.0, sb = 0.0;
+// Folds the [numParts, n2] fp32 partial rows into grad_weight (and grad_bias) in fp64.  A 256-thread group covers 32
+// consecutive columns (8 threads x 16 bytes = 128 bytes of a partial row) x 32 slices of the rows; a thread's loads of a
+// batch are independent and in flight together, so 512 partial rows are one round trip.  n2 is a multiple of 4.
+constexpr int kFoldCols = 32;
+constexpr int kFoldSlices = 256 / (kFoldCols / 4);
+template <typename T>
+__global__ __launch_bounds__(256) void rmsNormBwdFold(T* __restrict__ gradWeight, T* __restrict__ gradBias, const float* __restrict__ partW,
+                                                       const float* __restrict__ partB, int numParts, int n2) {
+    __shared__ double red[2][kFoldSlices][kFoldCols + 1];
+    const int c4 = threadIdx.x % (kFoldCols / 4);
+    const int slice = threadIdx.x / (kFoldCols / 4);
+    const int col = blockIdx.x * kFoldCols + c4 * 4;
+    double sw[4] = {0.0, 0.0, 0.0, 0.0}, sb[4] = {0.0, 0.0, 0.0, 0.0};
     if (col < n2) {
-        constexpr int kBatch = 16;  // loads of a batch are independent and in flight together: 256 partial rows are one round trip
-        for (int p0 = slice; p0 < numParts; p0 += kSlices * kBatch) {
-            ColAcc vw[kBatch], vb[kBatch];
+        constexpr int kBatch = 16;
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        for (int p0 = slice; p0 < numParts; p0 += kFoldSlices * kBatch) {
+            f32x4 vw[kBatch], vb[kBatch];
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                const int p = p0 + kSlices * u;
-                vw[u] = p < numParts ? partW[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
-                vb[u] = (gradBias != nullptr && p < numParts) ? partB[static_cast<int64_t>(p) * n2 + col] : ColAcc(0);
+                const int p = p0 + kFoldSlices * u;
+                vw[u] = p < numParts ? *reinterpret_cast<const f32x4*>(partW + static_cast<int64_t>(p) * n2 + col) : zero;
+                vb[u] = (gradBias != nullptr && p < numParts) ? *reinterpret_cast<const f32x4*>(partB + static_cast<int64_t>(p) * n2 + col) : zero;
             }
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
-                sw += static_cast<double>(vw[u]);
-                sb += static_cast<double>(vb[u]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sw[e] += static_cast<double>(vw[u][e]);
+                    sb[e] += static_cast<double>(vb[u][e]);
+                }
             }
         }
     }
-    red[0][slice][c] = sw;
-    red[1][slice][c] = sb;
-    __syncthreads();
-    if (slice == 0 && col < n2) {
-        sw = 0.0;
-        sb = 0.0;
 #pragma unroll
-        for (int k = 0; k < kSlices; ++k) {
-            sw += red[0][k][c];
-            sb += red[1][k][c];
-        }
-        gradWeight[col] = fromDouble<T>(sw);
-        if (gradBias != nullptr) gradBias[col] = fromDouble<T>(sb);
+    for (int e = 0; e < 4; ++e) {
+        red[0][slice][c4 * 4 + e] = sw[e];
+        red[1][slice][c4 * 4 + e] = sb[e];
+    }
+    __syncthreads();
+    // threads 0..31 finish grad_weight, 32..63 grad_bias: the slices in their fixed order
+    const int which = threadIdx.x / kFoldCols;
+    const int c = threadIdx.x % kFoldCols;
+    const int outCol = blockIdx.x * kFoldCols + c;
+    if (which < 2 && outCol < n2 && (which == 0 || gradBias != nullptr)) {
+        double sum = 0.0;
+#pragma unroll 8
+        for (int k = 0; k < kFoldSlices; ++k) sum += red[which][k][c];
+        (which == 0 ? gradWeight : gradBias)[outCol] = fromDouble<T>(sum);
     }
 }
 
@@ -662,12 +674,12 @@ diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const Tenso
 
 // Launches one instantiation of the fused backward kernel; the LDS column-sum arrays are dynamic shared memory
 // beyond the 64 KiB static limit, which has to be granted per kernel and device.
-template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS>
-diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, ColAcc* partW, ColAcc* partB, const T* dout, const T* in, const T* w,
+template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS, int WGS>
+diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, float* partW, float* partB, const T* dout, const T* in, const T* w,
                                const float* invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
     constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * kBwdTeam * EPV * sizeof(ColAcc);
-    auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS>;
+    auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS, WGS>;
     ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(kernel), static_cast<int>(ldsBytes)));
     hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2);
     ROCM_LAUNCH_CHECK();
@@ -681,45 +693,73 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     *launched = false;
     if (d.n2 % EPV != 0 || d.n2 > INT32_MAX) return diopiSuccess;
     const int64_t nvec = d.n2 / EPV;
-    // one team array is at most 32 KiB of LDS; four teams without grad_bias, two with (128 KiB per work-group)
-    constexpr int kMaxNvt = static_cast<int>(32768 / (kBwdTeam * EPV * sizeof(ColAcc)));
+    // The shape of the work-groups by the packets a thread holds per row (NVT), all within 128 KiB of LDS per compute unit
+    // (a team array is NVT * 256 packets of ColAcc).  Measured without grad_bias, main kernel alone:
+    //   fp32 [8192, 4096] (NVT 4): two groups of two teams 68.0 us, one group of four teams 71.4 us
+    //   fp32 [32768, 1024] (NVT 1): 67.5 against 63.4 us; bf16 [8192, 4096] (NVT 2): 37.8 against 36.7 us
+    //   bf16 [4096, 8192] (NVT 4): one group of two teams 46.3 us against 108.9 us for four teams, whose 16 waves leave a lane
+    //   128 registers where the kernel wants 217
+    // so fp32 NVT 4 takes two groups of two teams per unit, fewer packets one group of four; 16-bit NVT 4 (217 registers) and
+    // fp32 rows of up to 8192 columns (NVT 8, 64 KiB per team array, 236 registers) one group of two.  With grad_bias a team
+    // has two arrays: one group of two teams (one of one team at NVT 8).
+    constexpr int kMaxNvt = sizeof(T) == 4 ? 8 : 4;
     if (nvec > static_cast<int64_t>(kMaxNvt) * kBwdTeam) return diopiSuccess;
     if (deviceInfo().maxSharedOptin < 128 * 1024 + 1024) return diopiSuccess;
     if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
     const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
-    const int groups = gBias ? 2 : 4;
-    // one work-group per compute unit (fewer when there are not enough rows to give every team one)
-    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU);
+    const int nvc = nvt <= 1 ? 1 : (nvt <= 2 ? 2 : (nvt <= 4 ? 4 : 8));
+    // (fp32 NVT 4 with fewer than 16 rows per compute unit: one group of four again, 23.2 against 25.9 us at [2048, 4096], where
+    // the second partial row per unit costs more than the faster stream brings)
+    const bool twoPerUnit = !gBias && nvc == 4 && sizeof(T) == 4 && d.n1 >= 16 * static_cast<int64_t>(deviceInfo().numCU);
+    const int groups = gBias ? (nvc == 8 ? 1 : 2) : ((nvc <= 2 || (nvc == 4 && sizeof(T) == 4 && !twoPerUnit)) ? 4 : 2);
+    const int perUnit = twoPerUnit ? 2 : 1;
+    // as many work-groups as fit the compute units (fewer when there are not enough rows to give every team one)
+    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * perUnit;
     const int numParts = static_cast<int>(std::min<int64_t>(maxBlocks, ceilDiv(d.n1, groups)));
     const int n2 = static_cast<int>(d.n2);
-    const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(ColAcc);
+    const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(float);
     void* scratch = nullptr;
     ROCM_CALL(requireScratch(ctx, partBytes * (gBias ? 2 : 1), &scratch));
-    ColAcc* partW = static_cast<ColAcc*>(scratch);
-    ColAcc* partB = gBias ? partW + static_cast<int64_t>(numParts) * n2 : nullptr;
+    float* partW = static_cast<float*>(scratch);
+    float* partB = gBias ? partW + static_cast<int64_t>(numParts) * n2 : nullptr;
     T* pgi = static_cast<T*>(gIn.data);
     const T* pdo = static_cast<const T*>(dout.data);
     const T* pin = static_cast<const T*>(in.data);
     const T* pw = static_cast<const T*>(w.data);
     const float* pinv = static_cast<const float*>(invRms.data);
-#define ROCM_BWD_CASE(NVC)                                                                                                          \
-    if constexpr (NVC <= kMaxNvt) {                                                                                                 \
-        if (gBias != nullptr) {                                                                                                     \
-            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, true, 2>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)));  \
-        } else {                                                                                                                    \
-            ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, false, 4>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2))); \
-        }                                                                                                                           \
-    }
-    if (nvt <= 1) {
-        ROCM_BWD_CASE(1)
-    } else if (nvt <= 2) {
-        ROCM_BWD_CASE(2)
+#define ROCM_BWD_CASE(NVC, GB, GROUPS, WGS) \
+    ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, GB, GROUPS, WGS>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)))
+    if (gBias != nullptr) {
+        if (nvc == 1) {
+            ROCM_BWD_CASE(1, true, 2, 1);
+        } else if (nvc == 2) {
+            ROCM_BWD_CASE(2, true, 2, 1);
+        } else if (nvc == 4) {
+            ROCM_BWD_CASE(4, true, 2, 1);
+        } else if constexpr (kMaxNvt >= 8) {
+            ROCM_BWD_CASE(8, true, 1, 1);
+        }
     } else {
-        ROCM_BWD_CASE(4)
+        if (nvc == 1) {
+            ROCM_BWD_CASE(1, false, 4, 1);
+        } else if (nvc == 2) {
+            ROCM_BWD_CASE(2, false, 4, 1);
+        } else if (nvc == 4) {
+            if constexpr (sizeof(T) == 4) {
+                if (twoPerUnit) {
+                    ROCM_BWD_CASE(4, false, 2, 2);
+                } else {
+                    ROCM_BWD_CASE(4, false, 4, 1);
+                }
+            } else {
+                ROCM_BWD_CASE(4, false, 2, 1);
+            }
+        } else if constexpr (kMaxNvt >= 8) {
+            ROCM_BWD_CASE(8, false, 2, 1);
+        }
     }
 #undef ROCM_BWD_CASE
-    constexpr int kFoldCols = 128 / static_cast<int>(sizeof(ColAcc));
-    hipLaunchKernelGGL((rmsNormBwdFold<T, ColAcc>), dim3(static_cast<unsigned>(ceilDiv(n2, kFoldCols))), dim3(256), 0, stream, static_cast<T*>(gW.data),
+    hipLaunchKernelGGL((rmsNormBwdFold<T>), dim3(static_cast<unsigned>(ceilDiv(n2, kFoldCols))), dim3(256), 0, stream, static_cast<T*>(gW.data),
                        static_cast<T*>(gBias), partW, partB, numParts, n2);
     ROCM_LAUNCH_CHECK();
     *launched = true;

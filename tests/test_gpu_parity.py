@@ -197,7 +197,8 @@ def test_rms_norm_reference_cases(golden, dtype):
 
 
 @pytest.mark.parametrize("shape,dtype", [((512, 4096), "float32"), ((300, 4096), "bfloat16"), ((129, 8192), "float16"), ((64, 1024), "float32"),
-                                         ((33, 2048), "float16"), ((17, 4104), "float32"), ((8, 16384), "float32"), ((5, 40000), "float16")])
+                                         ((33, 2048), "float16"), ((17, 4104), "float32"), ((8, 16384), "float32"), ((5, 40000), "float16"), ((130, 8192), "float32"), ((1100, 6144), "float32"),
+                                         ((1030, 8192), "bfloat16")])
 def test_rms_norm_wide_rows(shape, dtype):
     say("rms_norm wide", shape, dtype)
     _rms_case(shape, (shape[-1],), 1e-6, TORCH_DTYPES[dtype], with_bias=(shape[0] % 2 == 1), seed=300, ones_grad=False)
