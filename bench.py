@@ -50,6 +50,89 @@ def measured_traffic(kernel, total_tokens):
     return None
 
 
+def token_attention_floor(args, torch, rt, W, impl, ctx, check):
+    """What the memory system charges for diopiTokenAttentionInference's access pattern at the cfg5 shape, without arithmetic.
+
+    Times, on the operator's own inputs and stream: the operator; a gather of the same cache rows through the same b_loc
+    windows (256-token tiles, one work-group each); the gather plus a write of the logits' volume cut into pieces of 256
+    bytes to 32 KiB per tile (512 bytes, one run per head, is the layout the interface prescribes); the writes alone; and a
+    plain copy of the same number of bytes.  Prints one JSON line per measurement."""
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(rt.IMPL_LIB_PATH), "libdiopi_probes.so"))
+    lib.diopiProbeTokenGather.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                          ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    lib.diopiProbeCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int]
+    dev = "cuda:0"
+    w = W.cfg5(dev, seed=5)
+    B, H, Hkv, D, total, mil = w["B"], w["H"], w["Hkv"], w["D"], w["total_len"], w["max_input_len"]
+    e = 2
+    row_bytes = Hkv * D * e
+    tile = 256
+    logits = torch.zeros(H, total, dtype=w["dtype"], device=dev)
+    h = {k: rt.Tensor(w[k]) for k in ("k_cache", "q", "b_loc", "b_seq_len", "b_start_loc")}
+    h["logits"] = rt.Tensor(logits)
+    assert w["b_loc"].dtype == torch.int32 and w["b_seq_len"].dtype == torch.int32 and w["b_start_loc"].dtype == torch.int32
+    stream = ctypes.c_void_p(ctx.torch_stream.cuda_stream)
+    max_len = int(w["b_seq_len"].max())
+    read_bytes = total * row_bytes
+    write_bytes = total * H * e
+    out = torch.zeros(write_bytes + 65536, dtype=torch.uint8, device=dev)
+    src = torch.zeros(read_bytes, dtype=torch.uint8, device=dev)
+    dst = torch.zeros(read_bytes, dtype=torch.uint8, device=dev)
+
+    def timed(fn, steps=args.steps, warmup=args.warmup):
+        for _ in range(warmup):
+            fn()
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < args.warm_seconds:
+            for _ in range(8):
+                fn()
+            ctx.synchronize()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(ctx)
+        for _ in range(steps):
+            fn()
+        e1.record(ctx)
+        ms = e0.elapsed_ms(e1)
+        ctx.synchronize()
+        return ms / steps * 1e3
+
+    def say(**kw):
+        print(json.dumps(kw), flush=True)
+
+    def gather(mode, pieces, split, tile=tile):
+        per_piece = (total * H * e // pieces + 15) // 16 * 16
+        r = lib.diopiProbeTokenGather(stream, mode, w["k_cache"].data_ptr(), row_bytes, w["b_loc"].data_ptr(), mil, w["b_start_loc"].data_ptr(),
+                                      w["b_seq_len"].data_ptr(), B, max_len, out.data_ptr(), per_piece, pieces, H * e, tile, split)
+        assert r == 0, "diopiProbeTokenGather refused its arguments"
+
+    say(probe="token-attention-floor", workload="cfg5 bf16 [B=%d, H=%d, Hkv=%d, D=%d]" % (B, H, Hkv, D), tokens=total, read_MB=round(read_bytes / 1e6, 1),
+        logits_MB=round(write_bytes / 1e6, 1), tile_tokens=tile, steps=args.steps)
+    us = timed(lambda: check(impl.diopiTokenAttentionInference(ctx.handle, h["logits"].handle, h["q"].handle, h["k_cache"].handle, h["b_loc"].handle,
+                                                               h["b_start_loc"].handle, h["b_seq_len"].handle, mil), "diopiTokenAttentionInference"))
+    say(what="diopiTokenAttentionInference", us=round(us, 1), GBs=round((read_bytes + write_bytes) / us / 1e3, 1))
+    # the read side alone, for each way of sharing a row between work-groups and each cache policy; the best one carries the writes
+    best = None
+    for split in (1, 2, 4, 8):
+        for nt in (0, 4):
+            for tt in (128, 256):
+                us = timed(lambda: gather(1 + nt, H, split, tt))
+                say(what="gather only", row_bytes_per_work_group=row_bytes // split, non_temporal=bool(nt), tile_tokens=tt, us=round(us, 1),
+                    GBs=round(read_bytes / us / 1e3, 1))
+                if tt == tile and (best is None or us < best[0]):
+                    best = (us, split, nt)
+    _, split, nt = best
+    for pieces in (2 * H, H, H // 2, H // 4, H // 16, 1):
+        piece_bytes = tile * H * e // pieces
+        us_both = timed(lambda: gather(3 + nt, pieces, split))
+        us_wr = timed(lambda: gather(2, pieces, split))
+        say(what="gather + logits-sized write", row_bytes_per_work_group=row_bytes // split, non_temporal=bool(nt), piece_bytes=piece_bytes,
+            interface_layout=(pieces == H), us=round(us_both, 1), GBs=round((read_bytes + write_bytes) / us_both / 1e3, 1), write_only_us=round(us_wr, 1))
+    wgs = 8 * int(rt.libs().rt.diopirtDeviceComputeUnits(0))
+    us = timed(lambda: lib.diopiProbeCopy(stream, dst.data_ptr(), src.data_ptr(), read_bytes, wgs))
+    say(what="plain copy of the read volume", us=round(us, 1), GBs=round(2 * read_bytes / us / 1e3, 1))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -58,6 +141,7 @@ def main():
     ap.add_argument("--no-diagnostic", action="store_true", help="skip the entries marked diagnostic (counter runs: they launch the same kernels on other data)")
     ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,penalty,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--probe", type=str, default="", help="instead of the benchmark, time a memory-pattern probe beside its operator: token-attention-floor")
     ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
     args = ap.parse_args()
@@ -104,6 +188,13 @@ def main():
 
     def check(ret, what):
         rt.check_returncode(ret, what)
+
+    if args.probe:
+        if args.probe != "token-attention-floor":
+            print("unknown probe %r (known: token-attention-floor)" % args.probe, file=sys.stderr)
+            sys.exit(2)
+        token_attention_floor(args, torch, rt, W, impl, ctx, check)
+        return
 
     class Timing(float):
         """Average milliseconds per step of one timed region, with the median and minimum over its blocks."""

@@ -1,0 +1,180 @@
+// Measurement probes for gfx950, built into lib/libdiopi_probes.so and called only by `bench.py --probe`: kernels that move
+// the bytes of an operator in the operator's access pattern and do no arithmetic, so that their time is the floor the memory
+// system sets for that pattern.  Not part of the operator library and not exported by it.
+//
+// diopiProbeTokenGather follows diopiTokenAttentionInference (reference semantics functions_lightllm.cpp:53-80): a
+// work-group owns a tile of `tileTokens` consecutive tokens of one sequence, looks their cache slots up in
+// b_loc[i, max_input_len - L_i + t] and reads the slots' rows (all kv heads of a token are `rowBytes` contiguous bytes); it
+// then writes tokens * bytesPerToken bytes, which is what the operator's logits [H, total tokens] take for the tile, cut into
+// `pieces` equal runs of consecutive bytes that lie `pieceStride` bytes apart (pieces = H is the operator's own layout: one
+// run per head; fewer pieces of more bytes each are what another output layout would give).  `rowSplit` work-groups share a
+// tile: each reads its 1/rowSplit of every row (the operator gives a work-group some of the kv heads) and writes every
+// rowSplit-th piece.  Modes: 1 reads only, 2 writes only, 3 both; + 4 makes the reads non-temporal.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kBatch = 8;  // loads a thread issues before it looks at the first of them; two such batches are in flight
+
+struct GatherArgs {
+    const char* cache;       // [slots][rowBytes]
+    const int32_t* loc;      // [batch][maxInputLen]
+    const int32_t* start;    // [batch] first token of the sequence in the output
+    const int32_t* length;   // [batch]
+    char* out;
+    int64_t pieceStride;     // bytes between the pieces of a tile
+    int rowBytes;            // 16 * a power of two, at most 4096
+    int partBytes;           // rowBytes / rowSplit: what one work-group reads of a row
+    int maxInputLen;
+    int tileTokens;
+    int pieces;
+    int bytesPerToken;       // output bytes a token stands for (all pieces together)
+    int mode;
+};
+
+template <bool NT>
+__global__ __launch_bounds__(kThreads) void probeTokenGather(GatherArgs a) {
+    // x runs over the parts of a row, y over the sequences, z over the tiles, with the sequence rotated by the tile index:
+    // work-groups that start together read neighbouring parts of the same rows and tiles of many sequences, and the
+    // thinly populated late tiles of the ragged batch come last
+    const int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    const int L = a.length[i];
+    const int t0 = blockIdx.z * a.tileTokens;
+    if (t0 >= L) return;
+    const int n = min(a.tileTokens, L - t0);
+    const int tid = threadIdx.x;
+    uint32_t acc = tid;
+    // the tile's slots go to LDS in one coalesced load, so that no row address waits for a load of its own
+    extern __shared__ int32_t slotOf[];
+    if (a.mode & 1) {
+        const int32_t* slots = a.loc + static_cast<int64_t>(i) * a.maxInputLen + (a.maxInputLen - L) + t0;
+        for (int t = tid; t < n; t += kThreads) slotOf[t] = slots[t];
+        __syncthreads();
+    }
+    if (a.mode & 1) {
+        const int packetsPerRow = a.partBytes / 16;
+        const int rowsPerStep = kThreads / packetsPerRow;  // token rows one load instruction of the work-group covers
+        const int rowSel = tid / packetsPerRow;
+        const int packet = tid % packetsPerRow;
+        const int steps = (n + rowsPerStep - 1) / rowsPerStep;
+        auto issue = [&](u32x4 (&buf)[kBatch], int s0) {
+#pragma unroll
+            for (int r = 0; r < kBatch; ++r) {
+                int t = (s0 + r) * rowsPerStep + rowSel;
+                t = t < n ? t : n - 1;  // past the tile: the last row again (a line that is already on its way)
+                const u32x4* p = reinterpret_cast<const u32x4*>(a.cache + static_cast<int64_t>(slotOf[t]) * a.rowBytes + blockIdx.x * a.partBytes + packet * 16);
+                buf[r] = NT ? __builtin_nontemporal_load(p) : *p;
+            }
+        };
+        auto take = [&](const u32x4 (&buf)[kBatch]) {
+#pragma unroll
+            for (int r = 0; r < kBatch; ++r) acc += buf[r].x ^ buf[r].y ^ buf[r].z ^ buf[r].w;
+        };
+        // every trip of the loop issues both batches (rows past the tile are the last row again): with no branch around a
+        // load the compiler knows how many are outstanding at each use and waits for just the oldest, instead of for all of
+        // them.  The scheduling barriers keep the order written here: without them the two uses are merged ahead of the two
+        // issues and one batch is in flight instead of two.
+        u32x4 b0[kBatch], b1[kBatch];
+        const int padded = (steps + 2 * kBatch - 1) / (2 * kBatch) * (2 * kBatch);
+        issue(b0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(b1, kBatch);
+        __builtin_amdgcn_sched_barrier(0);
+        for (int s = 2 * kBatch; s < padded; s += 2 * kBatch) {
+            take(b0);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(b0, s);
+            __builtin_amdgcn_sched_barrier(0);
+            take(b1);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(b1, s + kBatch);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        take(b0);
+        take(b1);
+    }
+    if (a.mode & 2) {
+        // the tile's output as 16-byte packets: piece p starts where the tile's first token lies in run p of the output
+        const int perTokenPerPiece = a.bytesPerToken / a.pieces;
+        const int packetsPerPiece = n * perTokenPerPiece / 16;
+        const int64_t first = (static_cast<int64_t>(a.start[i] + t0) * perTokenPerPiece) & ~int64_t(15);
+        const u32x4 v = {acc, acc + 1, acc + 2, acc + 3};
+        const int mine = (a.pieces - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);  // pieces x, x + rowSplit, ...
+        for (int q = tid; q < packetsPerPiece * mine; q += kThreads) {
+            const int p = (q / packetsPerPiece) * gridDim.x + blockIdx.x;
+            const int within = q % packetsPerPiece;
+            *reinterpret_cast<u32x4*>(a.out + p * a.pieceStride + first + within * 16) = v;
+        }
+    } else if (acc == 0x7fffffffu) {
+        *reinterpret_cast<uint32_t*>(a.out) = acc;  // keeps the loads alive; the value never occurs
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void probeCopy(u32x4* __restrict__ dst, const u32x4* __restrict__ src, int64_t packets) {
+    // four packets a thread in flight, each instruction of the work-group on 4 KiB of consecutive bytes; whole groups of four
+    // without a branch around a load, the rest one by one
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads * 4;
+    int64_t p0 = static_cast<int64_t>(blockIdx.x) * kThreads * 4 + threadIdx.x;
+    for (; p0 + 3 * kThreads < packets; p0 += stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(src + p0 + u * kThreads);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) __builtin_nontemporal_store(v[u], dst + p0 + u * kThreads);
+    }
+    for (int u = 0; u < 4; ++u) {
+        const int64_t p = p0 + u * kThreads;
+        if (p < packets) dst[p] = src[p];
+    }
+}
+
+}  // namespace
+
+// Launches one pass of the gather probe on `stream`.  Returns 0, or 1 when the arguments do not fit what the kernel assumes.
+extern "C" int diopiProbeTokenGather(void* stream, int mode, const void* cache, int rowBytes, const int32_t* loc, int maxInputLen, const int32_t* start,
+                                     const int32_t* length, int batch, int maxLength, void* out, int64_t pieceStride, int pieces, int bytesPerToken,
+                                     int tileTokens, int rowSplit) {
+    if (rowSplit <= 0 || rowBytes % rowSplit != 0) return 1;
+    const int partBytes = rowBytes / rowSplit;
+    const bool rowOk = partBytes >= 16 && partBytes <= 16 * kThreads && (partBytes & (partBytes - 1)) == 0;
+    if (!rowOk || (mode & 3) == 0 || mode > 7 || batch <= 0 || batch > 65535 || maxLength <= 0 || tileTokens <= 0 || pieces <= 0 || bytesPerToken % pieces != 0 ||
+        (tileTokens * (bytesPerToken / pieces)) % 16 != 0 || pieceStride % 16 != 0)
+        return 1;
+    GatherArgs a;
+    a.cache = static_cast<const char*>(cache);
+    a.loc = loc;
+    a.start = start;
+    a.length = length;
+    a.out = static_cast<char*>(out);
+    a.pieceStride = pieceStride;
+    a.rowBytes = rowBytes;
+    a.partBytes = partBytes;
+    a.maxInputLen = maxInputLen;
+    a.tileTokens = tileTokens;
+    a.pieces = pieces;
+    a.bytesPerToken = bytesPerToken;
+    a.mode = mode;
+    const dim3 grid(static_cast<unsigned>(rowSplit), static_cast<unsigned>(batch), static_cast<unsigned>((maxLength + tileTokens - 1) / tileTokens));
+    if (tileTokens > 8192) return 1;  // the slots of a tile in LDS
+    const size_t lds = static_cast<size_t>(tileTokens) * sizeof(int32_t);
+    if (mode & 4) {
+        hipLaunchKernelGGL(probeTokenGather<true>, grid, dim3(kThreads), lds, static_cast<hipStream_t>(stream), a);
+    } else {
+        hipLaunchKernelGGL(probeTokenGather<false>, grid, dim3(kThreads), lds, static_cast<hipStream_t>(stream), a);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// A plain copy of `bytes` bytes (a multiple of 16) with 16-byte accesses: the yardstick the counters and the stream rates are
+// read against.
+extern "C" int diopiProbeCopy(void* stream, void* dst, const void* src, int64_t bytes, int workGroups) {
+    if (bytes <= 0 || bytes % 16 != 0 || workGroups <= 0) return 1;
+    hipLaunchKernelGGL(probeCopy, dim3(static_cast<unsigned>(workGroups)), dim3(kThreads), 0, static_cast<hipStream_t>(stream), static_cast<u32x4*>(dst),
+                       static_cast<const u32x4*>(src), bytes / 16);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
