@@ -133,6 +133,67 @@ def token_attention_floor(args, torch, rt, W, impl, ctx, check):
     say(what="plain copy of the read volume", us=round(us, 1), GBs=round(2 * read_bytes / us / 1e3, 1))
 
 
+def matrix_rate(args, torch, rt, W, impl, ctx, check):
+    """The rate and the clock a loop of nothing but v_mfma_f32_32x32x16 products sustains on every compute unit (operands in
+    registers, finite non-trivial values), and diopiContextAttentionInference at cfg4 in the same process: the published
+    2.5 PFLOP/s is 1024 flop per clock and SIMD at 2.4 GHz; under a sustained matrix load the part runs slower."""
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(rt.IMPL_LIB_PATH), "libdiopi_probes.so"))
+    lib.diopiProbeMatrixRate.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 4
+    dev = "cuda:0"
+    cus = int(rt.libs().rt.diopirtDeviceComputeUnits(0))
+    stream = ctypes.c_void_p(ctx.torch_stream.cuda_stream)
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    iters = 40000  # 640 000 products per wave: about 10 ms
+
+    def say(**kw):
+        print(json.dumps(kw), flush=True)
+
+    say(probe="matrix-rate", compute_units=cus, products_per_wave=16 * iters, flop_per_product=32768)
+    for name, bf16 in (("f16", 0), ("bf16", 1)):
+        for waves in (4, 8):
+            clocks = torch.zeros(cus * waves * 2, dtype=torch.int64, device=dev)
+            for _ in range(3):  # the first launches bring the part to its sustained state
+                assert lib.diopiProbeMatrixRate(stream, clocks.data_ptr(), sink.data_ptr(), cus, waves, iters, bf16) == 0
+            ctx.synchronize()
+            e0, e1 = rt.Event(), rt.Event()
+            e0.record(ctx)
+            assert lib.diopiProbeMatrixRate(stream, clocks.data_ptr(), sink.data_ptr(), cus, waves, iters, bf16) == 0
+            e1.record(ctx)
+            ms = e0.elapsed_ms(e1)
+            ctx.synchronize()
+            c = clocks.cpu().view(-1, 2).double()
+            flop = cus * waves * iters * 16 * 32768.0
+            ghz = float((c[:, 0] / c[:, 1]).mean()) * 0.1
+            # pipe share: 32 clocks per product and SIMD over the shader clocks the slowest wave of a SIMD needed
+            per_simd = waves // 4
+            pipe = per_simd * iters * 16 * 32.0 / float(c[:, 0].max())
+            say(what="v_mfma_f32_32x32x16_" + name, waves_per_simd=per_simd, ms=round(ms, 3), TFLOPs=round(flop / ms / 1e9, 1),
+                shader_GHz=round(ghz, 3), matrix_pipe_busy=round(pipe, 3))
+    w4 = W.cfg4(dev, seed=4)
+    flops = W.context_attention_flops(w4["seq_len_host"], w4["H"], w4["D"])
+    for name, dt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        q, k, v = (w4[x].to(dt) for x in ("q", "k", "v"))
+        out = torch.zeros_like(q)
+        h = {n_: rt.Tensor(t) for n_, t in (("q", q), ("k", k), ("v", v), ("out", out), ("start", w4["b_start_loc"]), ("len", w4["b_seq_len"]))}
+
+        def call():
+            check(impl.diopiContextAttentionInference(ctx.handle, h["out"].handle, h["q"].handle, h["k"].handle, h["v"].handle, h["start"].handle,
+                                                      h["len"].handle, w4["max_input_len"]), "diopiContextAttentionInference")
+            ctx.clear_tensors()
+
+        for _ in range(args.warmup + 200):
+            call()
+        ctx.synchronize()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(ctx)
+        for _ in range(args.steps):
+            call()
+        e1.record(ctx)
+        ms = e0.elapsed_ms(e1) / args.steps
+        ctx.synchronize()
+        say(what="diopiContextAttentionInference cfg4 " + name, ms=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,7 +202,8 @@ def main():
     ap.add_argument("--no-diagnostic", action="store_true", help="skip the entries marked diagnostic (counter runs: they launch the same kernels on other data)")
     ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,penalty,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--probe", type=str, default="", help="instead of the benchmark, time a memory-pattern probe beside its operator: token-attention-floor")
+    ap.add_argument("--probe", type=str, default="", help="instead of the benchmark, run a probe: token-attention-floor (the memory cost of TokenAttention's access pattern at cfg5) "
+                    "or matrix-rate (what a loop of nothing but matrix products sustains, beside the prefill kernel at cfg4)")
     ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
     args = ap.parse_args()
@@ -190,10 +252,13 @@ def main():
         rt.check_returncode(ret, what)
 
     if args.probe:
-        if args.probe != "token-attention-floor":
-            print("unknown probe %r (known: token-attention-floor)" % args.probe, file=sys.stderr)
+        if args.probe == "token-attention-floor":
+            token_attention_floor(args, torch, rt, W, impl, ctx, check)
+        elif args.probe == "matrix-rate":
+            matrix_rate(args, torch, rt, W, impl, ctx, check)
+        else:
+            print("unknown probe %r (known: token-attention-floor, matrix-rate)" % args.probe, file=sys.stderr)
             sys.exit(2)
-        token_attention_floor(args, torch, rt, W, impl, ctx, check)
         return
 
     class Timing(float):

@@ -900,14 +900,22 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
         auto tooLow = [&]() -> bool { return __any(tm > kPipeLazyLog2); };
         int event = 0;
         if (jt < dg) {
+            // The wave's priority steps down with the phases.  Of two waves on a SIMD the instruction arbiter serves the older
+            // one first (in a loop of nothing but products it gets 85 % of the matrix pipe), so the four older waves of a
+            // group reach the next barrier 380 clocks before the four younger ones, which then run alone and less well.  With
+            // the steps, a wave that is a phase ahead ranks below its neighbour: 230 clocks, +0.5-1 % on the whole kernel.
             do {
                 top();
+                __builtin_amdgcn_s_setprio(3);
                 scores(Yes(), 0, s1, s0, early);  // phase 1
+                __builtin_amdgcn_s_setprio(2);
                 values(Yes(), 0, s1, tm, early);  // phase 2
+                __builtin_amdgcn_s_setprio(1);
                 if (tooLow()) {
                     event = 1;
                 } else {
                     scores(Yes(), 1, s0, s1, early);  // phase 3
+                    __builtin_amdgcn_s_setprio(0);
                     values(Yes(), 1, s0, tm, early);  // phase 4
                     flipK();
                     flipV();
@@ -916,6 +924,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
                     if (jt < dg && tooLow()) event = 2;
                 }
             } while (jt < dg && event == 0);
+            __builtin_amdgcn_s_setprio(0);
         }
         // the row's maximum over the 32 keys of half s; moves the reference when it is more than the lazy margin above it
         auto settleHalf = [&](f32x16& s) {

@@ -1,6 +1,7 @@
 // Measurement probes for gfx950, built into lib/libdiopi_probes.so and called only by `bench.py --probe`: kernels that move
 // the bytes of an operator in the operator's access pattern and do no arithmetic, so that their time is the floor the memory
-// system sets for that pattern.  Not part of the operator library and not exported by it.
+// system sets for that pattern, and a loop of nothing but matrix products, whose rate is what the matrix cores sustain at the
+// clock the power limit leaves them.  Not part of the operator library and not exported by it.
 //
 // diopiProbeTokenGather follows diopiTokenAttentionInference (reference semantics functions_lightllm.cpp:53-80): a
 // work-group owns a tile of `tileTokens` consecutive tokens of one sequence, looks their cache slots up in
@@ -133,7 +134,86 @@ __global__ __launch_bounds__(kThreads) void probeCopy(u32x4* __restrict__ dst, c
     }
 }
 
+// The rate the matrix cores sustain: every wave runs `iters` rounds of 16 v_mfma_f32_32x32x16 products (four accumulators,
+// operands held in registers) and leaves its shader-clock and 100 MHz-clock counts behind, so that the caller gets both the
+// product rate and the clock the part ran at.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <bool BF16>
+__global__ __launch_bounds__(512) void probeMatrixRate(long long* __restrict__ clocks, float* __restrict__ sink, int iters) {
+    const int lane = threadIdx.x % 64;
+    // operands: every 16-bit element gets a hashed sign and mantissa and an exponent that puts it in 1/32 .. 1/2 (the spread
+    // of attention operands: scaled queries and keys, probabilities), so that consecutive products, which take different
+    // operand registers, switch the multiplier inputs the way real data does
+    u32x4 raw[8];
+    for (int i = 0; i < 8; ++i) {
+        for (int c = 0; c < 4; ++c) {
+            uint32_t h = (static_cast<uint32_t>(lane) * 8u + i) * 4u + c;
+            h = (h ^ 61u) ^ (h >> 16);
+            h *= 9u;
+            h ^= h >> 4;
+            h *= 0x27d4eb2du;
+            h ^= h >> 15;
+            uint32_t lo, hi;
+            if (BF16) {
+                lo = (h & 0x807fu) | ((0x7au + ((h >> 8) & 3u)) << 7);
+                hi = ((h >> 16) & 0x807fu) | ((0x7au + ((h >> 24) & 3u)) << 7);
+            } else {
+                lo = (h & 0x83ffu) | ((0x0au + ((h >> 11) & 3u)) << 10);
+                hi = ((h >> 16) & 0x83ffu) | ((0x0au + ((h >> 27) & 3u)) << 10);
+            }
+            raw[i][c] = lo | (hi << 16);
+        }
+    }
+    f32x16 acc[4];
+    for (int j = 0; j < 4; ++j)
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+    const long long c0 = __builtin_amdgcn_s_memtime();
+    const long long w0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const int ia = (st + j) % 8, ib = (st + 2 * j + 4) % 8;
+                if constexpr (BF16) {
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw[ia]), __builtin_bit_cast(bf16x8, raw[ib]), acc[j], 0, 0, 0);
+                } else {
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, raw[ia]), __builtin_bit_cast(f16x8, raw[ib]), acc[j], 0, 0, 0);
+                }
+            }
+        }
+    }
+    const long long c1 = __builtin_amdgcn_s_memtime();
+    const long long w1 = __builtin_amdgcn_s_memrealtime();
+    float t = 0.f;
+    for (int j = 0; j < 4; ++j)
+        for (int r = 0; r < 16; ++r) t += acc[j][r];
+    if (t == 1.2345f) *sink = t;
+    if (lane == 0) {
+        long long* c = clocks + (static_cast<long long>(blockIdx.x) * (blockDim.x / 64) + threadIdx.x / 64) * 2;
+        c[0] = c1 - c0;
+        c[1] = w1 - w0;
+    }
+}
+
 }  // namespace
+
+// One launch of the matrix-rate probe: `workGroups` groups of `waves` waves (4 or 8: one or two per SIMD), `iters` rounds of
+// 16 products per wave.  clocks: [workGroups * waves][2] (shader clocks, 10 ns ticks) per wave; sink: 4 bytes.
+extern "C" int diopiProbeMatrixRate(void* stream, void* clocks, void* sink, int workGroups, int waves, int iters, int bf16) {
+    if (workGroups <= 0 || (waves != 4 && waves != 8) || iters <= 0) return 1;
+    if (bf16) {
+        hipLaunchKernelGGL(probeMatrixRate<true>, dim3(static_cast<unsigned>(workGroups)), dim3(static_cast<unsigned>(waves * 64)), 0,
+                           static_cast<hipStream_t>(stream), static_cast<long long*>(clocks), static_cast<float*>(sink), iters);
+    } else {
+        hipLaunchKernelGGL(probeMatrixRate<false>, dim3(static_cast<unsigned>(workGroups)), dim3(static_cast<unsigned>(waves * 64)), 0,
+                           static_cast<hipStream_t>(stream), static_cast<long long*>(clocks), static_cast<float*>(sink), iters);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : 1;
+}
 
 // Launches one pass of the gather probe on `stream`.  Returns 0, or 1 when the arguments do not fit what the kernel assumes.
 extern "C" int diopiProbeTokenGather(void* stream, int mode, const void* cache, int rowBytes, const int32_t* loc, int maxInputLen, const int32_t* start,
