@@ -51,7 +51,8 @@ def measured_traffic(kernel, total_tokens):
 
 
 def token_attention_floor(args, torch, rt, W, impl, ctx, check):
-    """What the memory system charges for diopiTokenAttentionInference's access pattern at the cfg5 shape, without arithmetic.
+    """What the memory system charges for diopiTokenAttentionInference's access pattern at the cfg5 shape (cfg3 with --only cfg3),
+    without arithmetic.
 
     Times, on the operator's own inputs and stream: the operator; a gather of the same cache rows through the same b_loc
     windows (256-token tiles, one work-group each); the gather plus a write of the logits' volume cut into pieces of 256
@@ -62,7 +63,8 @@ def token_attention_floor(args, torch, rt, W, impl, ctx, check):
                                           ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
     lib.diopiProbeCopy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int]
     dev = "cuda:0"
-    w = W.cfg5(dev, seed=5)
+    which = "cfg3" if "cfg3" in args.only else "cfg5"
+    w = W.cfg3(dev, seed=3) if which == "cfg3" else W.cfg5(dev, seed=5)
     B, H, Hkv, D, total, mil = w["B"], w["H"], w["Hkv"], w["D"], w["total_len"], w["max_input_len"]
     e = 2
     row_bytes = Hkv * D * e
@@ -106,14 +108,16 @@ def token_attention_floor(args, torch, rt, W, impl, ctx, check):
                                       w["b_seq_len"].data_ptr(), B, max_len, out.data_ptr(), per_piece, pieces, H * e, tile, split)
         assert r == 0, "diopiProbeTokenGather refused its arguments"
 
-    say(probe="token-attention-floor", workload="cfg5 bf16 [B=%d, H=%d, Hkv=%d, D=%d]" % (B, H, Hkv, D), tokens=total, read_MB=round(read_bytes / 1e6, 1),
+    say(probe="token-attention-floor", workload="%s %s [B=%d, H=%d, Hkv=%d, D=%d]" % (which, str(w["dtype"])[6:], B, H, Hkv, D), tokens=total, read_MB=round(read_bytes / 1e6, 1),
         logits_MB=round(write_bytes / 1e6, 1), tile_tokens=tile, steps=args.steps)
     us = timed(lambda: check(impl.diopiTokenAttentionInference(ctx.handle, h["logits"].handle, h["q"].handle, h["k_cache"].handle, h["b_loc"].handle,
                                                                h["b_start_loc"].handle, h["b_seq_len"].handle, mil), "diopiTokenAttentionInference"))
     say(what="diopiTokenAttentionInference", us=round(us, 1), GBs=round((read_bytes + write_bytes) / us / 1e3, 1))
     # the read side alone, for each way of sharing a row between work-groups and each cache policy; the best one carries the writes
     best = None
-    for split in (1, 2, 4, 8):
+    for split in (1, 2, 4, 8, 16, 32):
+        if row_bytes // split > 4096 or row_bytes // split < 256:
+            continue
         for nt in (0, 4):
             for tt in (128, 256):
                 us = timed(lambda: gather(1 + nt, H, split, tt))
