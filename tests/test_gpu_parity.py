@@ -970,6 +970,25 @@ def test_context_attention_config4_full_size_sampled():
     assert_close(o2, vconst, rtol=1e-2, atol=1e-3, what="cfg4 full, constant V")
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_context_attention_config4_full_size_two_kernels_agree(dtype):
+    """cfg4 at full size, every row of every head: the lightllm operator (the pipelined kernel) against
+    diopiFlashAttentionVarLen on the same tokens (the kernel's general form: another loop, cumulative lengths, its own
+    softmax-scale path).  Each is within 1e-2 of the exact result on the rows the oracle samples; here the whole tensors must
+    agree to a few roundings of the element type, which a wrong tile, half or row anywhere in either kernel would break."""
+    dt = TORCH_DTYPES[dtype]
+    w = W.cfg4(DEV, seed=4)
+    q, k, v = (w[x].to(dt) for x in ("q", "k", "v"))
+    out = torch.full_like(q, 55.0)
+    F.context_attention(q, k, v, out, w["b_start_loc"], w["b_seq_len"], w["max_input_len"])
+    cu = torch.cat((w["b_start_loc"], (w["b_start_loc"][-1:] + w["b_seq_len"][-1:]))).int()
+    flash = F.flash_attention_varlen(q, k, v, cu, cu, None, w["max_input_len"], w["max_input_len"], 0.0, None, True)
+    assert not torch.isnan(out).any() and not torch.isnan(flash).any()
+    tol = 2e-3 if dt is torch.float16 else 1.6e-2  # measured: 1.2e-4 in fp16, one bf16 step (7.8e-3) in bf16
+    assert_close(out, flash, rtol=tol, atol=tol, what=f"cfg4 full size {dtype}: lightllm prefill vs flash varlen")
+    say("cfg4 full size", dtype, "two kernels: max_abs/rel %.3e %.3e" % report(out.cpu(), flash.cpu()))
+
+
 # ----------------------------------------------------------------------------- variable-length flash attention
 # the reference's cases (diopi_configs.py:9854-9945): (q shape, key/value heads of the grouped case, cumulative lengths,
 # max_seqlen, is_causal, softmax_scale)
