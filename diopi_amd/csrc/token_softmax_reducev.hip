@@ -76,29 +76,17 @@ __device__ __forceinline__ float waveSumUniform(float v) {
     return (laneValue(v, 0) + laneValue(v, 16)) + (laneValue(v, 32) + laneValue(v, 48));
 }
 
-template <typename T, int GC>
-__global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
-                                                                    SplitArgs sp) {
-    using Ops = Mfma16<T>;
-    using Frag = typename Ops::Frag;
-    __shared__ __attribute__((aligned(16))) T sP[kRvWaves][GC * kTilePitch];
-    __shared__ __attribute__((aligned(16))) int32_t sSlotW[kRvWaves][kSub];
-    __shared__ __attribute__((aligned(16))) float sStat[kRvWaves][16];
-    __shared__ __attribute__((aligned(16))) float sMerge[kRvWaves][GC][kMergePitch];  // per wave and query head: 128 sums, maximum, denominator
-
-    // x runs over kv heads (neighbouring work-groups read neighbouring 256-byte pieces of the same cache rows at the same
-    // time), y and z over the (sequence, range) items
-    const int waveId = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    // Which (sequence, range) is this work-group's?  The one whose token count has the rank of the work-group's index
-    // (y, then z: the order in which work-groups start), over all items when there are at most 256, else over the
-    // sequences of each range (a range's token counts fall with the sequence length like the lengths themselves);
-    // with more sequences than that the items are taken as they come, the sequence rotated by the range so that
-    // neighbouring work-groups mix ranges of different sequences.
+// Which (sequence, range) is this work-group's?  The one whose token count has the rank of the work-group's index
+// (y, then z: the order in which work-groups start), over all items when there are at most 256, else over the
+// sequences of each range (a range's token counts fall with the sequence length like the lengths themselves);
+// with more sequences than that the items are taken as they come, the sequence rotated by the range so that
+// neighbouring work-groups mix ranges of different sequences.  Called by every thread of the work-group.
+__device__ __forceinline__ void rankedItem(const DecodeArgs& a, const SplitArgs& sp, int waveId, int& i, int& zIdx) {
     __shared__ int sItem;
     const int nSeq = static_cast<int>(gridDim.y);
     const int nRanges = static_cast<int>(gridDim.z);
-    int i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
-    int zIdx = static_cast<int>(blockIdx.z);
+    i = static_cast<int>((blockIdx.y + blockIdx.z) % gridDim.y);
+    zIdx = static_cast<int>(blockIdx.z);
     if (nSeq <= kRankedItems && nSeq * nRanges > 1) {  // at most 256 x 65535 items: no overflow
         if (waveId == 0) {
             auto lengthOf = [&](int seq) {
@@ -121,6 +109,23 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         i = sItem % nSeq;
         zIdx = sItem / nSeq;
     }
+}
+
+template <typename T, int GC>
+__global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restrict__ out, const T* __restrict__ logits, const T* __restrict__ v, DecodeArgs a,
+                                                                    SplitArgs sp) {
+    using Ops = Mfma16<T>;
+    using Frag = typename Ops::Frag;
+    __shared__ __attribute__((aligned(16))) T sP[kRvWaves][GC * kTilePitch];
+    __shared__ __attribute__((aligned(16))) int32_t sSlotW[kRvWaves][kSub];
+    __shared__ __attribute__((aligned(16))) float sStat[kRvWaves][16];
+    __shared__ __attribute__((aligned(16))) float sMerge[kRvWaves][GC][kMergePitch];  // per wave and query head: 128 sums, maximum, denominator
+
+    // x runs over kv heads (neighbouring work-groups read neighbouring 256-byte pieces of the same cache rows at the same
+    // time), y and z over the (sequence, range) items
+    const int waveId = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    int i, zIdx;
+    rankedItem(a, sp, waveId, i, zIdx);
     int64_t L = loadIndex(a.bSeqLen, i, a.len64);
     if (L > a.maxInputLen) L = a.maxInputLen;
     const int64_t t0 = static_cast<int64_t>(zIdx) * sp.TT;
