@@ -14,7 +14,10 @@
 //      h / (H / Hkv); fp32 scores and sums, probabilities rounded to the element type before the product with V
 //   5. inoutput[b, 0 : H*D] = out[b] (H*D <= hidden_units; columns past H*D keep their values)
 // Open in the prose, fixed here: the rotary pairing (2), a circular cache window once L reaches max_seq_len (3, 4),
-// where the output lands when H*D < hidden_units (5), and that finished rows are left untouched everywhere.
+// where the output lands when H*D < hidden_units (5), that finished rows are left untouched everywhere, and the caches'
+// dimensions: the header writes [num_layer, batch, local_head_num, max_seq_len, size_per_head]; a cache holds kv heads, so
+// dimension 2 is local_kv_head_num here, and dimension 1 may exceed this call's batch_size (an engine allocates for its
+// largest batch): the layer stride is taken from the caches themselves.
 //
 // Four kernels for 16-bit tensors with heads of 128 (three plain ones further down for everything else), all on the
 // context's stream:
