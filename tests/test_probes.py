@@ -113,3 +113,22 @@ def test_copy_and_matrix_rate_probes():
             # 800 products of 32 matrix-pipe clocks each (16 when two waves share a SIMD and overlap perfectly)
             assert (c[:, 0] >= 50 * 16 * 16).all() and (c[:, 1] > 0).all()
             assert float(sink.abs().sum()) == 0.0
+
+
+@pytest.mark.gpu
+@pytest.mark.timeout(600)
+def test_bench_probe_modes_run_and_print_json():
+    """`bench.py --probe ...` end to end in a child process: every line it prints is JSON and the expected entries are there."""
+    import json
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for mode, extra, needle in (("matrix-rate", [], "v_mfma_f32_32x32x16_f16"), ("token-attention-floor", ["--only", "cfg3"], "gather + logits-sized write")):
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--probe", mode, "--steps", "5", "--warmup", "2", "--warm-seconds", "0"] + extra,
+                           cwd=root, capture_output=True, text=True, timeout=500)
+        assert r.returncode == 0, r.stderr[-2000:]
+        lines = [json.loads(ln) for ln in r.stdout.splitlines() if ln.strip()]
+        assert lines and lines[0]["probe"] == mode
+        assert any(needle in str(ln.get("what", "")) for ln in lines), lines
+        for ln in lines[1:]:
+            assert ln.get("us", ln.get("ms", 0)) > 0
