@@ -577,7 +577,14 @@ struct MfmaInPlace<bf16_t> {
         asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
     }
 };
-__device__ __forceinline__ void mfmaSettle() { asm volatile("s_nop 7\n\ts_nop 3" ::: "memory"); }
+// The wait runs through the registers it is for: a read of them that only depended on the product could be scheduled ahead of
+// the wait itself (a maximum taken from a score tuple one product short moves the softmax reference too little, and a
+// probability past 2^16 leaves the 16-bit range).
+__device__ __forceinline__ void mfmaSettle(f32x16& a) { asm volatile("s_nop 7\n\ts_nop 3" : "+v"(a)); }
+__device__ __forceinline__ void mfmaSettle(f32x16& a, f32x16& b) { asm volatile("s_nop 7\n\ts_nop 3" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void mfmaSettle(f32x16& a, f32x16& b, f32x16& c, f32x16& d) {
+    asm volatile("s_nop 7\n\ts_nop 3" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
 
 // The lightllm prefill operator as one software-pipelined instruction stream per wave (fp16 / bf16, D == 128, causal).
 //
@@ -878,7 +885,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
     float early[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // exponentials of scores 0..7 of the half that is next in line
     if (active) {
         scores(No(), 1, s0, s0, early);
-        mfmaSettle();
+        mfmaSettle(s0);
         if (dg > 0) {  // the first half sets the reference
             float m = 0.f;
 #pragma unroll
@@ -928,7 +935,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
         }
         // the row's maximum over the 32 keys of half s; moves the reference when it is more than the lazy margin above it
         auto settleHalf = [&](f32x16& s) {
-            mfmaSettle();
+            mfmaSettle(s);
             float m = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) m = maxStep(s, i, m);
@@ -966,7 +973,8 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
         top();
         const bool both = (waveRowLo & 32) != 0;
         if (both) scores(No(), 0, s1, s1, unusedEarly);
-        mfmaSettle();  // also for the accumulators of the loop's last products
+        mfmaSettle(s0, s1);  // the masks below overwrite what the last products wrote
+        mfmaSettle(o[0], o[1], o[2], o[3]);
         const int key0 = dg * kBN;
         const int row = waveRowLo + n;
 #pragma unroll
@@ -997,7 +1005,7 @@ __global__ __launch_bounds__(NWV * kWave, NWV == 4 ? 2 : 1) void ctxAttnPipe(T* 
         }
         ++jt;
     }
-    mfmaSettle();
+    mfmaSettle(o[0], o[1], o[2], o[3]);
     for (; jt < numKeyTiles; ++jt) top();  // the other waves' remaining tiles: this wave only fetches its share
 
     // ---- normalise, transpose through LDS, write rows with 16-byte stores ----

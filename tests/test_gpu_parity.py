@@ -888,11 +888,14 @@ def test_context_attention_long_odd_lengths_whole_output():
                       f"two long sequences {dt}")
 
 
-def _rising_case(L, H, dt, profile, what):
+def _rising_case(L, H, dt, profile, what, support=slice(0, 128)):
     """Scores that climb along the sequence: q = a * u + noise, k_j = b_j * u + noise with u a unit vector, so that the
-    score of key j is about a * b_j (in powers of two after the softmax scale: `profile(j)`)."""
+    score of key j is about a * b_j (in powers of two after the softmax scale: `profile(j)`).  `support`: the head dims u
+    lives on (the last 16 are the last of the eight products a score is summed from)."""
     g = gen(604)
-    u = torch.ones(128) / math.sqrt(128.0)
+    u = torch.zeros(128)
+    u[support] = 1.0
+    u = u / u.norm()
     a = 8.0
     to_raw = math.sqrt(128.0) / math.log2(math.e)  # from powers of two to the unscaled dot product
     b = torch.tensor([profile(j) * to_raw / a for j in range(L)])
@@ -921,6 +924,24 @@ def test_context_attention_rising_scores_move_the_softmax_reference(dtype):
         _rising_case(L, 2, dt, lambda j: (40.0 if j >= 200 else 0.0) + (30.0 if j >= 457 else 0.0),
                      f"jumps at keys 200 (lower half of tile 3) and 457 L={L} {dtype}")
         _rising_case(L, 2, dt, lambda j: 30.0 * (j % 64 == 63) + 20.0 * (j // 64), f"staircase with spikes L={L} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_context_attention_second_rise_after_the_pipeline_was_left(dtype):
+    """A first rise of the scores makes a wave leave its pipelined loop; a second one, by more than the 16 bits of headroom a
+    16-bit probability has, then lands in the plain loop, in the upper half of a key tile, on each of the positions whose scores
+    are the first to be read after the products (a read that came too early once moved the reference too little: NaN rows).
+    Steps (every later key stays high) and isolated spikes, the second one 18-30 powers of two above the first, with the whole
+    score carried by the last 16 head dims, i.e. by the last of the eight products it is summed from."""
+    dt = TORCH_DTYPES[dtype]
+    last = slice(112, 128)
+    for pos in (0, 1, 2, 3, 6, 7, 12, 31):
+        second = 64 * 9 + 32 + pos
+        _rising_case(700, 1, dt, lambda j: (40.0 if j >= 100 else 0.0) + (30.0 if j >= second else 0.0), f"steps at 100 and {second} {dtype}", last)
+        _rising_case(700, 1, dt, lambda j: 21.0 * (j < 32) + 42.0 * (j == 120) + 60.2 * (j == second), f"spikes at 120 and {second} {dtype}", last)
+    # the shape the fault was found at: spikes deep in a long sequence, rows far below them
+    _rising_case(2600, 1, dt, lambda j: 21.0 * (j < 32) + 42.0 * (j == 696) + 60.2 * (j == 1766), f"spikes at 696 and 1766, L=2600 {dtype}", last)
+    _rising_case(1100, 2, dt, lambda j: 60.0 * j / 1100, f"steady climb on the last dims {dtype}", last)
 
 
 def test_context_attention_config4_scaled():
