@@ -787,6 +787,59 @@ def _whole_batch_decode_checks(w, logits, out, what):
     assert_bit_equal(l2, logits, what + ": relabelling the cache slots changes nothing")
 
 
+def test_decode_pair_random_shapes_against_float64_on_the_device():
+    """120 seeded random draws of batch, head grouping (1 to 16 query heads per kv head), ragged lengths (empty sequences among
+    them), dtype and the spread of q and k: TokenAttention against the scaled dot products in float64, SoftmaxReduceV against
+    the float64 softmax of the logits the first operator wrote (probabilities rounded to the element type, as the reference
+    does), both evaluated on the device."""
+    g = gen(913)
+
+    def pick(*vals):
+        return vals[int(torch.randint(len(vals), (1,), generator=g))]
+
+    for case in range(120):
+        Hkv, G = pick(1, 2, 3, 8), pick(1, 2, 4, 5, 8, 16)
+        H = Hkv * G
+        B = pick(1, 2, 5, 17, 64)
+        hi = pick(5, 70, 300, 1000, 2500, 5000, 9000)
+        lens = torch.randint(0 if pick(0, 1) else 1, hi + 1, (B,), generator=g)
+        dt = pick(torch.float16, torch.bfloat16)
+        std = pick(0.5, 1.0, 3.0)
+        maxlen = max(1, int(lens.max()))
+        slots = int(lens.sum()) + 64
+        kc = (torch.randn(slots, Hkv, 128, generator=g) * std).to(dt).to(DEV)
+        vc = torch.randn(slots, Hkv, 128, generator=g).to(dt).to(DEV)
+        q = (torch.randn(B, H, 128, generator=g) * std).to(dt).to(DEV)
+        perm = torch.randperm(slots, generator=g)
+        b_loc = torch.zeros(B, maxlen, dtype=torch.int32)
+        start = torch.zeros(B, dtype=torch.int32)
+        pos = 0
+        for i, L in enumerate(lens.tolist()):
+            b_loc[i, maxlen - L:] = perm[pos:pos + L].int()
+            start[i] = pos
+            pos += L
+        total = max(1, pos)
+        b_loc, start, ln = b_loc.to(DEV), start.to(DEV), lens.int().to(DEV)
+        what = f"random decode case {case}: B={B} H={H} Hkv={Hkv} lengths {lens.tolist()[:8]} {dt} spread {std}"
+        logits = torch.full((H, total), -77.0, dtype=dt, device=DEV)
+        F.token_attention(q, kc, logits, b_loc, start, ln, maxlen)
+        out = torch.full_like(q, 5.0)
+        F.token_softmax_reducev(logits, vc, out, b_loc, start, ln, maxlen, 0)
+        assert bool(torch.isfinite(out.float()).all()), what + ": non-finite output"
+        for i, L in enumerate(lens.tolist()):
+            if L == 0:
+                assert int(out[i].count_nonzero()) == 0, what + ": an empty sequence gives zeros"
+                continue
+            sl = b_loc[i, maxlen - L:].long()
+            kk = kc[sl].double().repeat_interleave(G, dim=1)
+            vv = vc[sl].double().repeat_interleave(G, dim=1)
+            sc = torch.einsum("hd,lhd->hl", q[i].double(), kk) / math.sqrt(128.0)
+            got = logits[:, int(start[i]):int(start[i]) + L]
+            assert_close(got, sc, rtol=2e-2, atol=1e-2, what=what + f": logits of sequence {i}")  # two roundings to the element type
+            p = got.double().softmax(-1).to(dt).double()
+            assert_close(out[i], torch.einsum("hl,lhd->hd", p, vv), what=what + f": output of sequence {i}", **TOL[dt])
+
+
 def test_decode_config5_full_size_sampled():
     w = W.cfg5(DEV, seed=5)
     lens = w["b_seq_len"].tolist()
@@ -942,6 +995,53 @@ def test_context_attention_second_rise_after_the_pipeline_was_left(dtype):
     # the shape the fault was found at: spikes deep in a long sequence, rows far below them
     _rising_case(2600, 1, dt, lambda j: 21.0 * (j < 32) + 42.0 * (j == 696) + 60.2 * (j == 1766), f"spikes at 696 and 1766, L=2600 {dtype}", last)
     _rising_case(1100, 2, dt, lambda j: 60.0 * j / 1100, f"steady climb on the last dims {dtype}", last)
+
+
+def test_context_attention_random_shapes_two_kernels_and_float64():
+    """160 seeded random draws of batch, ragged lengths (with lengths on and next to the tile sizes), heads, dtype and the spread
+    of q and k (up to three times the configured one: sharply peaked softmax rows).  The lightllm operator must agree with
+    diopiFlashAttentionVarLen on the same tokens (another kernel) to a few roundings, both must be finite, and for modest sizes
+    both must match a float64 statement evaluated on the device.  bf16 draws with the widest spread are only checked for finite
+    results: there the reference's own composition is 0.19 off float64 (rounded scores of size 40 move probabilities by 10 %)."""
+    g = gen(911)
+
+    def pick(*vals):
+        return vals[int(torch.randint(len(vals), (1,), generator=g))]
+
+    for case in range(160):
+        B = pick(1, 2, 3, 5, 8, 12)
+        hi = pick(3, 40, 130, 300, 700, 1500, 3000)
+        lens = torch.randint(1, hi + 1, (B,), generator=g)
+        if pick(0, 1):
+            lens[int(torch.randint(B, (1,), generator=g))] = pick(1, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1024, 1025)
+        H = pick(1, 2, 5, 8)
+        dt = pick(torch.float16, torch.bfloat16)
+        std = pick(0.5, 1.0, 3.0)
+        T = int(lens.sum())
+        q = (torch.randn(T, H, 128, generator=g) * std).to(dt).to(DEV)
+        k = (torch.randn(T, H, 128, generator=g) * std).to(dt).to(DEV)
+        v = torch.randn(T, H, 128, generator=g).to(dt).to(DEV)
+        start = torch.cat((torch.zeros(1, dtype=torch.long), lens.cumsum(0)[:-1])).int().to(DEV)
+        ln = lens.int().to(DEV)
+        what = f"random prefill case {case}: lengths {lens.tolist()}, {H} heads, {dt}, spread {std}"
+        out = torch.full_like(q, 7.0)
+        F.context_attention(q, k, v, out, start, ln, int(lens.max()))
+        cu = torch.cat((start, (start[-1:] + ln[-1:]))).int()
+        flash = F.flash_attention_varlen(q, k, v, cu, cu, None, int(lens.max()), int(lens.max()), 0.0, None, True)
+        assert bool(torch.isfinite(out.float()).all()) and bool(torch.isfinite(flash.float()).all()), what + ": non-finite output"
+        if dt is torch.bfloat16 and std > 2:
+            continue
+        tol = 4e-3 if dt is torch.float16 else 2e-2
+        assert_close(out, flash, rtol=tol, atol=tol, what=what + ": the two kernels")
+        if T <= 4000 and std < 2:
+            s0 = 0
+            for L in lens.tolist():
+                qq, kk, vv = (t[s0:s0 + L].double().transpose(0, 1) for t in (q, k, v))
+                sc = qq @ kk.transpose(1, 2) / math.sqrt(128.0)
+                sc = sc.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool, device=DEV), 1), float("-inf"))
+                ref = (sc.softmax(-1) @ vv).transpose(0, 1)
+                assert_close(out[s0:s0 + L], ref, what=what + " vs float64 on the device", **TOL[dt])
+                s0 += L
 
 
 def test_context_attention_config4_scaled():
