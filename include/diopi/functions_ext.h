@@ -164,6 +164,10 @@ DIOPI_API diopiError_t diopiContextAttentionInferenceNoAlloc(diopiContextHandle_
  * the reference's statement; it is not read).  attention_out = softmax(softmax_scale * q k^T [+ causal mask]) v,
  * softmax_lse [batch, Hq, max_seqlen_q] (float32, may be null) receives the log-sum-exp of every query row's scaled
  * scores; entries past a sequence's length are left untouched.  softmax_scale == 0 means 1/sqrt(D).
+ * With float16 tensors at D == 128 the query is multiplied by the scale once and rounded to float16 (2^-11 relative);
+ * the output and softmax_lse both belong to those scores, so softmax_lse can differ from the log-sum-exp of unrounded
+ * scores by about 2^-12 of the largest scaled score of a row (5e-3 at a score of 35).  bfloat16 and float32 tensors scale
+ * every score in float32 instead.
  * Not implemented (error 13): p_dropout != 0, alibi_slopes, sliding windows (window sizes >= 0).  gen is not used.
  * dtypes: float16, bfloat16 (matrix cores at D == 128), float32, float64; cum_seq int32 or int64.
  */
