@@ -1885,6 +1885,70 @@ def test_c_host_runs_operators_through_the_c_abi():
 
 
 # ----------------------------------------------------------------------------- error behaviour on a GPU box
+def _strided_view(t):
+    big = torch.zeros(*t.shape[:-1], t.shape[-1] * 2, dtype=t.dtype, device=t.device)
+    view = big[..., ::2]
+    view.copy_(t)
+    return view
+
+
+def test_every_operator_refuses_strided_views_instead_of_reading_them_as_dense():
+    # impl/torch follows any stride through ATen; these kernels address rows by shape alone, so a view that is not densely
+    # packed must come back as an error from every entry point and every tensor argument (the adaptor's `contiguous: True`
+    # makes the copies).  The one exception is by design: diopiRotaryEmbedding follows the strides of cos and sin.
+    g = gen(1234)
+    B, H, D, T = 2, 4, 128, 6
+    lens = [4, 2]
+
+    def R(*shape):
+        return torch.randn(*shape, generator=g).half().to(DEV)
+
+    def I(values, dt=torch.int32):
+        return torch.tensor(values, dtype=dt, device=DEV)
+
+    loc = [[0, 1, 2, 3], [0, 0, 4, 5]]
+    cases = {
+        "rms_norm": (lambda x, w: F.rms_norm(x, (256,), w, None, 1e-6), [R(5, 256), R(256)]),
+        "rms_norm_backward": (lambda go, x, w: F.rms_norm_backward([go], x, w, None, (256,), 1e-6, inv_rms=torch.ones(5, 1, device=DEV)), [R(5, 256), R(5, 256), R(256)]),
+        "root_mean_square_norm_inp": (lambda x, w: F.root_mean_square_norm_inp(x, w, 1e-6), [R(5, 256), R(256)]),
+        "fused_add_root_mean_square_norm_inp": (lambda x, r, b, w: F.fused_add_root_mean_square_norm_inp(x, r, b, w, 1e-6), [R(5, 256), R(5, 256), R(256), R(256)]),
+        "rotary_emb": (lambda x: F.rotary_emb(x, R(T, 1, D // 2), R(T, 1, D // 2), False, False), [R(T, H, D)]),
+        "rotary_emb_v2": (lambda q, k, c, s: F.rotary_emb_v2(q, k, c, s, D), [R(T, H * D), R(T, H * D), R(T, 1, D), R(T, 1, D)]),
+        "apply_penalty": (lambda lg, p, f, ids, cnt, cum: F.apply_penalty(lg, p, f, ids, cnt, cum, 3),
+                          [R(2, 50), R(2), R(2), I([1, 2, 3, 4]), I([1, 1, 2, 2]), I([0, 3, 4])]),
+        "apply_penalty_v2": (lambda lg, p, f, r, ids, cnt: F.apply_penalty_v2(lg, p, f, r, ids, cnt), [R(2, 50), R(4), R(4), R(4), I([1, 2, 53, 54]), I([1, 1, 2, 2])]),
+        "destindex_copy_kv": (lambda k, dst, out: F.destindex_copy_kv(k, dst, out), [R(3, H, D), I([0, 5, 2]), R(8, H, D)]),
+        "token_attention": (lambda q, k, out, bl, bs, bq: F.token_attention(q, k, out, bl, bs, bq, 4), [R(B, H, D), R(16, H, D), R(H, 6), I(loc), I([0, 4]), I(lens)]),
+        "token_softmax_reducev": (lambda lg, v, out, bl, bs, bq: F.token_softmax_reducev(lg, v, out, bl, bs, bq, 4, 0),
+                                  [R(H, 6), R(16, H, D), R(B, H, D), I(loc), I([0, 4]), I(lens)]),
+        "context_attention": (lambda q, k, v, out, bs, bq: F.context_attention(q, k, v, out, bs, bq, 4),
+                              [R(T, H, D), R(T, H, D), R(T, H, D), R(T, H, D), I([0, 4]), I(lens)]),
+        "context_attention_no_alloc": (lambda q, k, v, out, bs, bq: F.context_attention_no_alloc(q, k, v, out, bs, bq, 4),
+                                       [R(T, H, D), R(T, H, D), R(T, H, D), R(T, H, D), I([0, 4]), I(lens)]),
+        "flash_attention_varlen": (lambda q, k, v, cu: F.flash_attention_varlen(q, k, v, cu, cu, None, 4, 4, 0, None, True),
+                                   [R(T, H, D), R(T, H, D), R(T, H, D), I([0, 4, 6])]),
+        "flash_attention": (lambda q, k, v: F.flash_attention(q, k, v, None, 0, None, True), [R(2, 3, H, D), R(2, 3, H, D), R(2, 3, H, D)]),
+        "multihead_attention": (lambda q, k, v: F.multihead_attention(q, k, v, 0, True, False, None), [R(2, 3, H, D), R(2, 3, H, D), R(2, 3, H, D)]),
+        "multihead_attention_varlen": (lambda q, k, v, cu: F.multihead_attention_varlen(q, k, v, cu, 4, 0, True, False, None),
+                                       [R(T, H, D), R(T, H, D), R(T, H, D), I([0, 4, 6], torch.int64)]),
+        "prompt_flash_attention": (lambda q, k, v: F.prompt_flash_attention(q, k, v, None, [3, 3], 3, H, H, D), [R(T, H * D), R(T, H * D), R(T, H * D)]),
+        "paged_attention": (lambda q, k, v, bt: F.paged_attention(q, k, v, None, lens, H, H, D, bt, 4), [R(B, H * D), R(16, H * D), R(16, H * D), I([[0, 1], [2, 3]])]),
+    }
+    for name, (call, tensors) in cases.items():
+        call(*[t.clone() for t in tensors])  # the dense call is valid
+        for i in range(len(tensors)):
+            args = [t.clone() for t in tensors]
+            args[i] = _strided_view(args[i])
+            assert not args[i].is_contiguous()
+            with pytest.raises(rt.DiopiException, match="contiguous"):
+                call(*args)
+    # the exception: strided cos / sin tables give the result of the dense ones
+    x, cos, sin = R(T, H, D), R(T, 1, D // 2), R(T, 1, D // 2)
+    assert_bit_equal(F.rotary_emb(x, _strided_view(cos), _strided_view(sin), False, False).cpu(), F.rotary_emb(x, cos, sin, False, False).cpu(),
+                     "rotary_emb follows the strides of cos and sin")
+    torch.cuda.synchronize()
+
+
 def test_errors_do_not_launch():
     x = torch.randn(4, 8, device=DEV)
     w = torch.ones(8, device=DEV)
