@@ -218,6 +218,13 @@ def test_fused_decoder_attention_far_positions():
     _case(B=3, H=4, Hkv=2, S=40, seq=[5, 39, 0], dt=torch.float32, seed=52, pad=[0, 7, 50000], step=100001, D=64, rot=64, what="position 1e5, float32")
 
 
+def test_fused_decoder_attention_long_caches():
+    # caches of 40000 to 70000 positions, nearly full, next to a short and an empty history; the plain kernels on 50000
+    _case(2, 8, 2, 40000, [39998, 12345], torch.float16, 5, hidden=1024, layers=1, layer=0, what="long cache fp16")
+    _case(3, 4, 4, 70000, [69999, 0, 35000], torch.bfloat16, 6, hidden=512, layers=1, layer=0, what="long cache bf16", step=70001)
+    _case(1, 16, 1, 50000, [49999], torch.float32, 7, hidden=1024, layers=1, layer=0, what="long cache fp32, plain kernels", D=64, rot=32)
+
+
 def test_fused_decoder_attention_more_items_than_the_ranking_takes():
     # 200 rows x 2 ranges of 1024 tokens are 400 items per kv head: past the 256 that are taken longest first, the plain order
     g = torch.Generator().manual_seed(61)

@@ -840,6 +840,52 @@ def test_decode_pair_random_shapes_against_float64_on_the_device():
             assert_close(out[i], torch.einsum("hl,lhd->hd", p, vv), what=what + f": output of sequence {i}", **TOL[dt])
 
 
+@pytest.mark.parametrize("Hkv,G,lens,dtype,index_dtype", [
+    (1, 16, [70001, 3, 20000], torch.bfloat16, torch.int64),
+    (8, 8, [33000, 1, 66000, 0, 127], torch.float16, torch.int32),
+    (2, 4, [262144], torch.bfloat16, torch.int32),
+])
+def test_decode_pair_very_long_sequences(Hkv, G, lens, dtype, index_dtype):
+    """Contexts far beyond the benchmark's (up to 262144 tokens: 32 or more ranges per sequence, the merge kernel's batches of 8
+    more than once) next to very short and empty ones, against float64 on the device in chunks of 16384 tokens."""
+    g = gen(915)
+    H, B = Hkv * G, len(lens)
+    maxlen, slots = max(lens), sum(lens) + 64
+    kc = torch.randn(slots, Hkv, 128, generator=g).to(dtype).to(DEV)
+    vc = torch.randn(slots, Hkv, 128, generator=g).to(dtype).to(DEV)
+    q = torch.randn(B, H, 128, generator=g).to(dtype).to(DEV)
+    perm = torch.randperm(slots, generator=g)
+    b_loc = torch.zeros(B, maxlen, dtype=index_dtype)
+    start = torch.zeros(B, dtype=index_dtype)
+    pos = 0
+    for i, L in enumerate(lens):
+        b_loc[i, maxlen - L:] = perm[pos:pos + L].to(index_dtype)
+        start[i] = pos
+        pos += L
+    b_loc, start, ln = b_loc.to(DEV), start.to(DEV), torch.tensor(lens, dtype=index_dtype, device=DEV)
+    logits = torch.full((H, pos), -77.0, dtype=dtype, device=DEV)
+    F.token_attention(q, kc, logits, b_loc, start, ln, maxlen)
+    out = torch.full_like(q, 5.0)
+    F.token_softmax_reducev(logits, vc, out, b_loc, start, ln, maxlen, 0)
+    for i, L in enumerate(lens):
+        what = f"long decode Hkv={Hkv} G={G} {dtype}: sequence {i} of {L} tokens"
+        if L == 0:
+            assert int(out[i].count_nonzero()) == 0, what + ": an empty sequence gives zeros"
+            continue
+        sl = b_loc[i, maxlen - L:].long()
+        got = logits[:, int(start[i]):int(start[i]) + L]
+        p = got.double().softmax(-1).to(dtype).double()
+        ref = torch.zeros(H, 128, dtype=torch.float64, device=DEV)
+        for c0 in range(0, L, 16384):
+            rows = sl[c0:c0 + 16384]
+            kk = kc[rows].double().repeat_interleave(G, dim=1)
+            vv = vc[rows].double().repeat_interleave(G, dim=1)
+            sc = torch.einsum("hd,lhd->hl", q[i].double(), kk) / math.sqrt(128.0)
+            assert_close(got[:, c0:c0 + 16384], sc, rtol=2e-2, atol=1e-2, what=what + f": logits from token {c0}")
+            ref += torch.einsum("hl,lhd->hd", p[:, c0:c0 + 16384], vv)
+        assert_close(out[i], ref, what=what + ": output", **TOL[dtype])
+
+
 def test_decode_config5_full_size_sampled():
     w = W.cfg5(DEV, seed=5)
     lens = w["b_seq_len"].tolist()
@@ -1042,6 +1088,30 @@ def test_context_attention_random_shapes_two_kernels_and_float64():
                 ref = (sc.softmax(-1) @ vv).transpose(0, 1)
                 assert_close(out[s0:s0 + L], ref, what=what + " vs float64 on the device", **TOL[dt])
                 s0 += L
+
+
+@pytest.mark.parametrize("B,longest,H,dtype", [(4200, 40, 2, torch.float16), (20000, 5, 1, torch.float16), (4000, 300, 1, torch.bfloat16)])
+def test_context_attention_thousands_of_short_sequences(B, longest, H, dtype):
+    """More sequences than the planning kernel of the matrix-core path keeps in LDS (the call then takes the one-wave-per-row
+    kernel), empty ones among them, and a batch just under that bound: every row against float64 on the device."""
+    g = gen(917)
+    lens = torch.randint(0, longest + 1, (B,), generator=g)
+    T = int(lens.sum())
+    q, k, v = (torch.randn(T, H, 128, generator=g).to(dtype).to(DEV) for _ in range(3))
+    start = torch.cat((torch.zeros(1, dtype=torch.long), lens.cumsum(0)[:-1])).int().to(DEV)
+    ln = lens.int().to(DEV)
+    out = torch.full_like(q, 7.0)
+    F.context_attention(q, k, v, out, start, ln, longest)
+    steps = torch.arange(longest, device=DEV)
+    valid = steps[None, :] < ln.long()[:, None]
+    rows = torch.where(valid, start.long()[:, None] + steps[None, :], torch.zeros_like(valid, dtype=torch.long))
+    causal = torch.tril(torch.ones(longest, longest, dtype=torch.bool, device=DEV))[None, None]
+    for b0 in range(0, B, 1000):
+        ii, live = rows[b0:b0 + 1000], valid[b0:b0 + 1000]
+        sc = torch.einsum("bthd,bshd->bhts", q[ii].double(), k[ii].double()) / math.sqrt(128.0)
+        sc = sc.masked_fill(~(causal & live[:, None, None, :]), float("-inf"))
+        ref = torch.einsum("bhts,bshd->bthd", sc.softmax(-1).nan_to_num(0.0), v[ii].double())
+        assert_close(out[ii][live], ref[live], what=f"{B} sequences of up to {longest} rows, {dtype}: sequences from {b0}", **TOL[dtype])
 
 
 def test_context_attention_config4_scaled():
