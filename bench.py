@@ -198,6 +198,99 @@ def matrix_rate(args, torch, rt, W, impl, ctx, check):
         say(what="diopiContextAttentionInference cfg4 " + name, ms=round(ms, 4), TFLOPs=round(flops / ms / 1e9, 1))
 
 
+# Child process of the sustained-clock probe: reads the board's shader clock (and power, where the tool reports it) twice a
+# second with rocm-smi and prints "unix_time MHz watts" lines until its standard input closes.  Started before the parent
+# touches the GPU; it never opens the device itself.
+CLOCK_SAMPLER = r"""
+import re, select, subprocess, sys, time
+while not select.select([sys.stdin], [], [], 0.5)[0]:
+    try:
+        txt = subprocess.run(["rocm-smi", "--showclocks", "--showpower"], capture_output=True, text=True, timeout=10).stdout
+    except Exception:
+        continue
+    clk = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", txt)
+    pw = re.search(r"Power \(W\): ([0-9.]+)", txt)
+    if clk:
+        print(time.time(), clk.group(1), pw.group(1) if pw else "nan", flush=True)
+"""
+
+
+def sustained_clock(args, torch, rt, W, impl, ctx, check, sampler):
+    """What shader clock the board holds while one operator runs back to back (--probe-seconds each, 7 by default): the prefill operator at
+    cfg4 on fp16 tensors, on bf16 tensors and on all-zero tensors, and the two decode operators at cfg3.  The readings come
+    from rocm-smi in a child process; a JSON line per workload with the median of the readings taken after the first 2 s."""
+    from diopi_amd.runtime import Tensor
+    dev = "cuda:0"
+    phases = []
+
+    def run(name, call, seconds=args.probe_seconds):
+        for _ in range(20):
+            call()
+        ctx.synchronize()
+        t0 = time.time()
+        n = 0
+        while time.time() - t0 < seconds:
+            for _ in range(200):
+                call()
+            ctx.synchronize()
+            n += 200
+        t1 = time.time()
+        phases.append((name, t0, t1, (t1 - t0) / n * 1e3))
+
+    w4 = W.cfg4(dev, seed=4)
+    flops = W.context_attention_flops(w4["seq_len_host"], w4["H"], w4["D"])
+    hs, hl = Tensor(w4["b_start_loc"]), Tensor(w4["b_seq_len"])
+    for name, make in (("diopiContextAttentionInference cfg4 fp16", lambda t: t), ("diopiContextAttentionInference cfg4 tokens in bf16", lambda t: t.to(torch.bfloat16)),
+                       ("diopiContextAttentionInference cfg4 shape, all-zero tensors", torch.zeros_like)):
+        q, k, v = (make(w4[n]) for n in ("q", "k", "v"))
+        o = torch.zeros_like(q)
+        h = {n: Tensor(t) for n, t in dict(q=q, k=k, v=v, o=o).items()}
+
+        def prefill():
+            check(impl.diopiContextAttentionInference(ctx.handle, h["o"].handle, h["q"].handle, h["k"].handle, h["v"].handle, hs.handle, hl.handle,
+                                                      w4["max_input_len"]), "diopiContextAttentionInference")
+            ctx.clear_tensors()
+
+        run(name, prefill)
+    del w4, q, k, v, o, h
+    torch.cuda.empty_cache()
+    w3 = W.cfg3(dev, seed=3)
+    logits = torch.zeros(w3["H"], w3["total_len"], dtype=w3["dtype"], device=dev)
+    out = torch.zeros_like(w3["q"])
+    h3 = {n: Tensor(w3[n]) for n in ("k_cache", "v_cache", "q", "b_loc", "b_seq_len", "b_start_loc")}
+    hlg, hout = Tensor(logits), Tensor(out)
+
+    def decode():
+        check(impl.diopiTokenAttentionInference(ctx.handle, hlg.handle, h3["q"].handle, h3["k_cache"].handle, h3["b_loc"].handle, h3["b_start_loc"].handle,
+                                                h3["b_seq_len"].handle, w3["max_input_len"]), "diopiTokenAttentionInference")
+        check(impl.diopiTokenSoftmaxReduceVInference(ctx.handle, hout.handle, hlg.handle, h3["v_cache"].handle, h3["b_loc"].handle, h3["b_start_loc"].handle,
+                                                     h3["b_seq_len"].handle, w3["max_input_len"], 0), "diopiTokenSoftmaxReduceVInference")
+        ctx.clear_tensors()
+
+    run("diopiTokenAttentionInference + diopiTokenSoftmaxReduceVInference cfg3", decode)
+    sampler.stdin.close()
+    readings = []
+    for ln in sampler.stdout:
+        parts = ln.split()
+        if len(parts) == 3:
+            readings.append((float(parts[0]), float(parts[1]), float(parts[2])))
+    sampler.wait(timeout=30)
+    nominal = int(rt.libs().rt.diopirtDeviceClockKHz(0)) / 1000.0
+    print(json.dumps(dict(probe="sustained-clock", source="rocm-smi --showclocks --showpower, two readings a second from a child process",
+                          device_max_clock_MHz=nominal, readings_total=len(readings))), flush=True)
+    for name, t0, t1, ms in phases:
+        mine = sorted(r for r in readings if t0 + 2.0 <= r[0] <= t1)
+        clk = sorted(r[1] for r in mine)
+        pw = sorted(r[2] for r in mine if r[2] == r[2])
+        e = dict(what=name, ms_per_call=round(ms, 4), readings=len(clk), sclk_MHz_median=clk[len(clk) // 2] if clk else None,
+                 sclk_MHz_min=clk[0] if clk else None, sclk_MHz_max=clk[-1] if clk else None, power_W_median=pw[len(pw) // 2] if pw else None)
+        if "ContextAttention" in name:
+            e["TFLOPs"] = round(flops / ms / 1e9, 1)
+            if clk:
+                e["fraction_of_max_clock"] = round(clk[len(clk) // 2] / nominal, 3)
+        print(json.dumps(e), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -207,7 +300,9 @@ def main():
     ap.add_argument("--only", type=str, default="", help="comma-separated subset of cfg1,cfg2,penalty,cfg3,cfg4,cfg5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--probe", type=str, default="", help="instead of the benchmark, run a probe: token-attention-floor (the memory cost of TokenAttention's access pattern at cfg5) "
-                    "or matrix-rate (what a loop of nothing but matrix products sustains, beside the prefill kernel at cfg4)")
+                    "matrix-rate (what a loop of nothing but matrix products sustains, beside the prefill kernel at cfg4) or sustained-clock (the shader clock the board "
+                    "holds under the prefill and decode operators, read with rocm-smi)")
+    ap.add_argument("--probe-seconds", type=float, default=7.0, help="sustained-clock: how long each workload runs (the first 2 s of readings are dropped)")
     ap.add_argument("--warm-seconds", type=float, default=WARM_SECONDS, help="untimed load before every timed region, on top of --warmup")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the headline CPU baseline sample")
     args = ap.parse_args()
@@ -215,6 +310,11 @@ def main():
         print("bench.py measures one GPU: every operator here is a single-device kernel and nothing in this build "
               "uses a second GPU (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+
+    sampler = None
+    if args.probe == "sustained-clock":  # the reader of the board's clock starts before this process touches the GPU
+        import subprocess
+        sampler = subprocess.Popen([sys.executable, "-c", CLOCK_SAMPLER], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
 
     import torch
 
@@ -260,8 +360,10 @@ def main():
             token_attention_floor(args, torch, rt, W, impl, ctx, check)
         elif args.probe == "matrix-rate":
             matrix_rate(args, torch, rt, W, impl, ctx, check)
+        elif args.probe == "sustained-clock":
+            sustained_clock(args, torch, rt, W, impl, ctx, check, sampler)
         else:
-            print("unknown probe %r (known: token-attention-floor, matrix-rate)" % args.probe, file=sys.stderr)
+            print("unknown probe %r (known: token-attention-floor, matrix-rate, sustained-clock)" % args.probe, file=sys.stderr)
             sys.exit(2)
         return
 

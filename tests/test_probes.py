@@ -123,7 +123,8 @@ def test_bench_probe_modes_run_and_print_json():
     import subprocess
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    for mode, extra, needle in (("matrix-rate", [], "v_mfma_f32_32x32x16_f16"), ("token-attention-floor", ["--only", "cfg3"], "gather + logits-sized write")):
+    for mode, extra, needle in (("matrix-rate", [], "v_mfma_f32_32x32x16_f16"), ("token-attention-floor", ["--only", "cfg3"], "gather + logits-sized write"),
+                                ("sustained-clock", ["--probe-seconds", "3.5"], "all-zero tensors")):
         r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--probe", mode, "--steps", "5", "--warmup", "2", "--warm-seconds", "0"] + extra,
                            cwd=root, capture_output=True, text=True, timeout=500)
         assert r.returncode == 0, r.stderr[-2000:]
@@ -131,4 +132,6 @@ def test_bench_probe_modes_run_and_print_json():
         assert lines and lines[0]["probe"] == mode
         assert any(needle in str(ln.get("what", "")) for ln in lines), lines
         for ln in lines[1:]:
-            assert ln.get("us", ln.get("ms", 0)) > 0
+            assert ln.get("us", ln.get("ms", ln.get("ms_per_call", 0))) > 0
+        if mode == "sustained-clock":  # the board's clock was read while every workload ran, and it never exceeds the device's maximum by more than a step
+            assert all(ln["readings"] >= 1 and 100 < ln["sclk_MHz_median"] <= lines[0]["device_max_clock_MHz"] + 50 for ln in lines[1:]), lines
