@@ -15,7 +15,7 @@
 //                                       x[r,l]   <- T(float(T(s)) * (inv * float(scale[l])))
 //
 // Layout: inoutput and residual [tokens, hidden] dense, scale and bias [hidden]; bias may be a null handle.
-// One 256-thread group owns a row and keeps it in registers as 16-byte packets, so every element is read once and
+// One group of 256 threads (512 with the residual addition) owns a row and keeps it in registers as 16-byte packets, so every element is read once and
 // written once: 2 (alone) or 4 (fused) passes over the matrix, which is what bounds the operator.  Many short-lived
 // groups, each touching one contiguous row, is the launch shape the memory system sustains its highest rate for.
 // Rows that do not fit that form (length not a multiple of a packet, more than 4 packets per thread, unaligned base)
@@ -28,14 +28,19 @@
 namespace rocm {
 namespace {
 
-constexpr int kRowThreads = 256;
+constexpr int kRowThreads = 256;  // threads of a group of the wave-per-row kernel, and of a row's group in the plain form
 constexpr int kRowWaves = kRowThreads / kWave;
+// Threads that own a row.  The plain form keeps the 256 of diopiRMSNorm's kernel, so that the two sum a row's squares in the
+// same order and give the same bits; with the residual addition 256 / 512 / 1024 measured 86.4 / 84.3 / 86.0 us at bf16
+// [16384, 4096].
+constexpr int rowThreads(bool fuseAdd) { return fuseAdd ? 512 : 256; }
 
 template <typename T, int NVT, bool FUSE_ADD, bool HAS_BIAS>
-__global__ __launch_bounds__(kRowThreads) void rmsNormInpBlockRow(T* __restrict__ inout, T* __restrict__ residual, const T* __restrict__ bias,
-                                                                   const T* __restrict__ scale, int64_t rows, int n, float eps) {
+__global__ __launch_bounds__(rowThreads(FUSE_ADD)) void rmsNormInpBlockRow(T* __restrict__ inout, T* __restrict__ residual, const T* __restrict__ bias,
+                                                                            const T* __restrict__ scale, int64_t rows, int n, float eps) {
     constexpr int EPV = Pack16<T>::N;
-    __shared__ float red[kRowWaves];
+    constexpr int kThreads = rowThreads(FUSE_ADD);
+    __shared__ float red[kThreads / kWave];
     const int tid = threadIdx.x;
     const int lane = tid % kWave;
     const int wave = tid / kWave;
@@ -48,7 +53,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsNormInpBlockRow(T* __restrict_
     Pack16<T> xv[NVT], rv[FUSE_ADD ? NVT : 1];
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-        const int v = j * kRowThreads + tid;
+        const int v = j * kThreads + tid;
         if (v < nvec) {
             xv[j] = loadPackStream(xr + v * EPV);
             if constexpr (FUSE_ADD) rv[j] = loadPackStream(rr + v * EPV);
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsNormInpBlockRow(T* __restrict_
     Pack16<T> sv[NVT], bv[HAS_BIAS ? NVT : 1];
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-        const int v = j * kRowThreads + tid;
+        const int v = j * kThreads + tid;
         if (v < nvec) {
             sv[j] = loadPack(scale + v * EPV);
             if constexpr (HAS_BIAS) bv[j] = loadPack(bias + v * EPV);
@@ -67,7 +72,7 @@ __global__ __launch_bounds__(kRowThreads) void rmsNormInpBlockRow(T* __restrict_
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-        const int v = j * kRowThreads + tid;
+        const int v = j * kThreads + tid;
         if (v < nvec) {
             if constexpr (FUSE_ADD) {
                 Pack16<T> nr;
@@ -94,12 +99,12 @@ __global__ __launch_bounds__(kRowThreads) void rmsNormInpBlockRow(T* __restrict_
     __syncthreads();
     float tot = 0.f;
 #pragma unroll
-    for (int i = 0; i < kRowWaves; ++i) tot += red[i];
+    for (int i = 0; i < kThreads / kWave; ++i) tot += red[i];
     const float inv = 1.0f / sqrtf(tot / static_cast<float>(n) + eps);
 
 #pragma unroll
     for (int j = 0; j < NVT; ++j) {
-        const int v = j * kRowThreads + tid;
+        const int v = j * kThreads + tid;
         if (v < nvec) {
             Pack16<T> o;
 #pragma unroll
@@ -161,7 +166,8 @@ diopiError_t launchTyped(hipStream_t stream, void* inout, void* residual, const 
     const T* pb = static_cast<const T*>(bias);
     const T* ps = static_cast<const T*>(scale);
     const int64_t nvec = n / EPV;
-    const bool fast = n % EPV == 0 && nvec <= 4 * kRowThreads && rows <= INT32_MAX && aligned16(inout) && aligned16(residual) && aligned16(bias) &&
+    constexpr int kThreads = rowThreads(FUSE_ADD);
+    const bool fast = n % EPV == 0 && nvec <= 4 * kThreads && rows <= INT32_MAX && aligned16(inout) && aligned16(residual) && aligned16(bias) &&
                       aligned16(scale);
     if (!fast) {
         int64_t blocks = ceilDiv(rows, kRowWaves);
@@ -171,14 +177,14 @@ diopiError_t launchTyped(hipStream_t stream, void* inout, void* residual, const 
         ROCM_LAUNCH_CHECK();
         return diopiSuccess;
     }
-    const int nvt = static_cast<int>(ceilDiv(nvec, kRowThreads));
+    const int nvt = static_cast<int>(ceilDiv(nvec, kThreads));
     const dim3 grid(static_cast<unsigned>(rows));
     const int ni = static_cast<int>(n);
 #define ROCM_INP_CASE(NVC)                                                                                                                        \
     if (FUSE_ADD && bias != nullptr) {                                                                                                            \
-        hipLaunchKernelGGL((rmsNormInpBlockRow<T, NVC, FUSE_ADD, FUSE_ADD>), grid, dim3(kRowThreads), 0, stream, px, pr, pb, ps, rows, ni, eps);   \
+        hipLaunchKernelGGL((rmsNormInpBlockRow<T, NVC, FUSE_ADD, FUSE_ADD>), grid, dim3(kThreads), 0, stream, px, pr, pb, ps, rows, ni, eps);   \
     } else {                                                                                                                                      \
-        hipLaunchKernelGGL((rmsNormInpBlockRow<T, NVC, FUSE_ADD, false>), grid, dim3(kRowThreads), 0, stream, px, pr, pb, ps, rows, ni, eps);      \
+        hipLaunchKernelGGL((rmsNormInpBlockRow<T, NVC, FUSE_ADD, false>), grid, dim3(kThreads), 0, stream, px, pr, pb, ps, rows, ni, eps);      \
     }
     if (nvt <= 1) {
         ROCM_INP_CASE(1)

@@ -12,8 +12,9 @@
 // Two kernels:
 //  * rotaryRows: the LLaMA layout.  x is viewed as [outer, A, B, D]; cos/sin are dense [A, D/2]
 //    tables shared by the B heads of a position (and by every `outer` slice).  A lane owns one
-//    16-byte packet position of the half-row and walks several heads with it, so cos/sin are
-//    fetched once per lane and every global access is a 128-bit one.
+//    16-byte packet position of the half-row of one head (kHeadsPerLane heads; one measured
+//    fastest: short-lived lanes with two loads of x in flight each), so every global access is a
+//    128-bit one and the small tables come from the cache.
 //  * rotaryGeneric: any right-aligned broadcast of cos/sin, element by element.
 #include "common.hpp"
 #include "device.hpp"
@@ -22,7 +23,7 @@ namespace rocm {
 namespace {
 
 constexpr int kRotThreads = 256;
-constexpr int kHeadsPerLane = 4;
+constexpr int kHeadsPerLane = 1;  // heads a lane rotates with one pair of table packets: 1 / 2 / 4 / 8 measured 85.4 / 86.3 / 89.0 / 90.1 us at [16384, 32, 128] bf16 x 2 tensors
 
 template <typename T>
 __device__ __forceinline__ void rotatePair(float x1, float x2, float c, float s, bool conj, T* o1, T* o2) {

@@ -10,9 +10,10 @@
 // Products and the sum are formed in fp32 (fp64 for fp64 tensors) and rounded once; the Python statement rounds each
 // product and the sum in the tensor dtype, which differs by at most two roundings of the element type.
 //
-// Kernel: a lane owns one 16-byte packet position p of the half-row (dims p*EPV .. +EPV-1 and the same + dim/2), keeps
-// the four table packets of its token in registers and walks four heads of query/key with them: every global access is
-// a 128-bit one and the tables are read once per lane.  Shapes that do not fit take an element-wise kernel.
+// Kernel: a lane owns one 16-byte packet position p of the half-row (dims p*EPV .. +EPV-1 and the same + dim/2) of one
+// head of query or key and reads the four table packets of its token for it (the tables are small and stay in cache): every
+// global access is a 128-bit one, and a lane has two loads of the tensor in flight, not more, which is what the memory
+// system streams fastest here (see kRot2HeadsPerLane).  Shapes that do not fit take an element-wise kernel.
 #include "common.hpp"
 #include "device.hpp"
 
@@ -20,7 +21,7 @@ namespace rocm {
 namespace {
 
 constexpr int kRot2Threads = 256;
-constexpr int kRot2HeadsPerLane = 4;
+constexpr int kRot2HeadsPerLane = 1;  // heads a lane rotates with one pair of table packets: 1 / 2 / 4 measured 83.1 / 88.7 / 91.0 us at [16384, 32, 128] bf16, query and key
 
 template <typename T>
 __device__ __forceinline__ T* headRow(T* q, T* k, int64_t t, int h, int hq, int hk, int dim) {
