@@ -259,11 +259,12 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 
 // ---------------------------------------------------------------------------
 // Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
-// A work-group is GROUPS row teams of 256 threads, WGS of them resident on a compute unit.  In step i, team g of work-group b takes row
+// A work-group is GROUPS row teams of TEAM threads (256, or 512 for fp32 rows of 1024 packets), one work-group per compute
+// unit.  In step i, team g of work-group b takes row
 // (i * gridDim.x + b) * GROUPS + g: at any moment the whole grid works on one contiguous window of
 // gridDim.x * GROUPS rows of each tensor, which spreads the traffic evenly over the memory channels (a private run of
 // rows per work-group would put the work-groups, which advance in step, a fixed large stride apart).
-// Thread t of a team owns packets t, t+256, ... of every row its team visits.
+// Thread t of a team owns packets t, t+TEAM, ... of every row its team visits.
 //
 // Rows travel through buffer loads and stores whose descriptor covers exactly one row (and nothing for a row past
 // the end of the work-group's run): packets beyond the row read as zero and stores to them are dropped by the
@@ -276,15 +277,13 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 // The column sums for grad_weight / grad_bias are accumulated in fp32 registers and moved every kBwdFlush steps into
 // per-team LDS arrays of ColAcc (fp64 for fp32 tensors), which bounds the length of any fp32 summation; at the end
 // the team arrays are summed in a fixed order into one fp32 partial row per work-group (one rounding of a sum that the
-// fold then continues in fp64: the error stays below one rounding of the fp32 result).  Without grad_bias a compute
-// unit holds two work-groups of two teams: the same 16 waves and 128 KiB of LDS as one work-group of four teams, but
-// the row stream runs 5 % faster that way (6.07 against 5.79 TB/s at fp32 [8192, 4096] with the partial rows and the
-// fold taken out of both builds; the barrier is not the reason, a build without it runs at the same speed), which pays
-// for the second partial row per unit once the partial rows are fp32.  The row sum s[r] crosses the team's four waves
-// through LDS: one barrier per step.
+// fold then continues in fp64: the error stays below one rounding of the fp32 result).  The fewer packets of a row a thread
+// holds, the faster the rows stream: at fp32 [8192, 4096] one work-group of four 256-thread teams (4 packets a thread)
+// moves the rows at 5.79 TB/s, two work-groups of two such teams per unit at 6.07, and one work-group of two 512-thread
+// teams (2 packets a thread, one partial row per unit) is another 2.5 % faster over the whole operator.  The row sum s[r]
+// crosses the team's waves through LDS: one barrier per step.
 // ---------------------------------------------------------------------------
-constexpr int kBwdTeam = 256;
-constexpr int kBwdTeamWaves = kBwdTeam / kWave;
+constexpr int kBwdTeam = 256;  // threads of a team unless a shape asks for more
 constexpr int kBwdFlush = 8;
 constexpr int kBufferWord3 = 0x00020000;  // raw buffer, 32-bit data format
 constexpr int kBufferStream = 2;          // cache policy: non-temporal
@@ -294,20 +293,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rowBuffer(const T* base, int64
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base + row * n2), 0, valid ? n2 * static_cast<int>(sizeof(T)) : 0, kBufferWord3);
 }
 
-// WGS work-groups of GROUPS teams share a compute unit: GROUPS * WGS waves on each of its four SIMDs, which is what the
-// second launch bound states (and what sets the registers a lane may use).
-template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS, int WGS>
-__global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused(T* __restrict__ gradInput, float* __restrict__ partW, float* __restrict__ partB,
+// A work-group is GROUPS teams of TEAM threads (256 or 512), one work-group per compute unit: GROUPS * TEAM / 256 waves on
+// each of its four SIMDs, which is what the second launch bound states (and what sets the registers a lane may use).
+template <typename T, typename ColAcc, int NVT, bool HAS_GBIAS, int GROUPS, int TEAM>
+__global__ __launch_bounds__(TEAM* GROUPS, GROUPS*(TEAM / 256)) void rmsNormBwdFused(T* __restrict__ gradInput, float* __restrict__ partW, float* __restrict__ partB,
                                                                        const T* __restrict__ dout, const T* __restrict__ x, const T* __restrict__ weight,
                                                                        const float* __restrict__ invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
-    constexpr int kCols = NVT * kBwdTeam * EPV;  // columns covered by the register tiling
-    __shared__ float red[2][GROUPS][kBwdTeamWaves];
+    constexpr int kCols = NVT * TEAM * EPV;  // columns covered by the register tiling
+    __shared__ float red[2][GROUPS][(TEAM / kWave)];
     extern __shared__ __attribute__((aligned(16))) unsigned char dynLds[];
     // [array(W,B)][team][(j*EPV + e)][tid]: lanes of a wave hit consecutive words
     ColAcc* sAcc = reinterpret_cast<ColAcc*>(dynLds);
-    const int team = __builtin_amdgcn_readfirstlane(threadIdx.x / kBwdTeam);  // the same for all lanes of a wave
-    const int tid = threadIdx.x % kBwdTeam;
+    const int team = __builtin_amdgcn_readfirstlane(threadIdx.x / TEAM);  // the same for all lanes of a wave
+    const int tid = threadIdx.x % TEAM;
     const int lane = tid % kWave;
     const int wave = tid / kWave;
     ColAcc* myW = sAcc + team * kCols;
@@ -327,7 +326,7 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
         const __amdgpu_buffer_rsrc_t bd = rowBuffer(dout, row, n2, valid);
 #pragma unroll
         for (int j = 0; j < NVT; ++j) {
-            const int off = (j * kBwdTeam + tid) * 16;
+            const int off = (j * TEAM + tid) * 16;
             r.x[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bx, off, 0, kBufferStream);
             r.d[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bd, off, 0, kBufferStream);
         }
@@ -339,7 +338,7 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
     {
         const __amdgpu_buffer_rsrc_t bw = rowBuffer(weight, 0, n2, true);
 #pragma unroll
-        for (int j = 0; j < NVT; ++j) wv[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bw, (j * kBwdTeam + tid) * 16, 0, 0);
+        for (int j = 0; j < NVT; ++j) wv[j].raw = __builtin_amdgcn_raw_buffer_load_b128(bw, (j * TEAM + tid) * 16, 0, 0);
     }
     RowRegs ra, rb;
     request(ra, rowOf(0));
@@ -354,8 +353,8 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
                 w[j][e] = toFloat(wv[j].e[e]);
                 accW[j][e] = 0.f;
                 if (HAS_GBIAS) accB[j][e] = 0.f;
-                myW[(j * EPV + e) * kBwdTeam + tid] = 0;
-                if (HAS_GBIAS) myB[(j * EPV + e) * kBwdTeam + tid] = 0;
+                myW[(j * EPV + e) * TEAM + tid] = 0;
+                if (HAS_GBIAS) myB[(j * EPV + e) * TEAM + tid] = 0;
             }
         }
     }
@@ -365,10 +364,10 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
         for (int j = 0; j < NVT; ++j) {
 #pragma unroll
             for (int e = 0; e < EPV; ++e) {
-                myW[(j * EPV + e) * kBwdTeam + tid] += static_cast<ColAcc>(accW[j][e]);
+                myW[(j * EPV + e) * TEAM + tid] += static_cast<ColAcc>(accW[j][e]);
                 accW[j][e] = 0.f;
                 if (HAS_GBIAS) {
-                    myB[(j * EPV + e) * kBwdTeam + tid] += static_cast<ColAcc>(accB[j][e]);
+                    myB[(j * EPV + e) * TEAM + tid] += static_cast<ColAcc>(accB[j][e]);
                     accB[j][e] = 0.f;
                 }
             }
@@ -397,7 +396,7 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
         __syncthreads();
         float sum2 = 0.f;
 #pragma unroll
-        for (int k = 0; k < kBwdTeamWaves; ++k) sum2 += red[i & 1][team][k];
+        for (int k = 0; k < (TEAM / kWave); ++k) sum2 += red[i & 1][team][k];
         const float term1 = (1.0f / fH) * inv;
         const __amdgpu_buffer_rsrc_t bg = rowBuffer(gradInput, row, n2, row < n1);
 #pragma unroll
@@ -412,7 +411,7 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
                 f *= term1;
                 gv.e[e] = fromFloat<T>(f);
             }
-            __builtin_amdgcn_raw_buffer_store_b128(gv.raw, bg, (j * kBwdTeam + tid) * 16, 0, kBufferStream);
+            __builtin_amdgcn_raw_buffer_store_b128(gv.raw, bg, (j * TEAM + tid) * 16, 0, kBufferStream);
         }
         request(r, rowOf(i + 2));
         if ((i % kBwdFlush) == kBwdFlush - 1) flush();
@@ -430,11 +429,11 @@ __global__ __launch_bounds__(kBwdTeam* GROUPS, GROUPS* WGS) void rmsNormBwdFused
 
     // one partial row per work-group: the team arrays are added in team order
     __syncthreads();
-    for (int idx = threadIdx.x; idx < kCols; idx += kBwdTeam * GROUPS) {
+    for (int idx = threadIdx.x; idx < kCols; idx += TEAM * GROUPS) {
         // idx = (j*EPV + e)*256 + t  <->  column (j*256 + t)*EPV + e
-        const int t = idx % kBwdTeam;
-        const int je = idx / kBwdTeam;
-        const int col = ((je / EPV) * kBwdTeam + t) * EPV + (je % EPV);
+        const int t = idx % TEAM;
+        const int je = idx / TEAM;
+        const int col = ((je / EPV) * TEAM + t) * EPV + (je % EPV);
         if (col < n2) {
             ColAcc sw = 0, sb = 0;
 #pragma unroll
@@ -674,14 +673,14 @@ diopiError_t forwardTyped(hipStream_t stream, const TensorView& out, const Tenso
 
 // Launches one instantiation of the fused backward kernel; the LDS column-sum arrays are dynamic shared memory
 // beyond the 64 KiB static limit, which has to be granted per kernel and device.
-template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS, int WGS>
+template <typename T, typename ColAcc, int NVT, bool GB, int GROUPS, int TEAM = kBwdTeam>
 diopiError_t launchBwdInstance(hipStream_t stream, int numParts, T* gIn, float* partW, float* partB, const T* dout, const T* in, const T* w,
                                const float* invRms, int64_t n1, int n2) {
     constexpr int EPV = Pack16<T>::N;
-    constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * kBwdTeam * EPV * sizeof(ColAcc);
-    auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS, WGS>;
+    constexpr size_t ldsBytes = static_cast<size_t>(GB ? 2 : 1) * GROUPS * NVT * TEAM * EPV * sizeof(ColAcc);
+    auto kernel = rmsNormBwdFused<T, ColAcc, NVT, GB, GROUPS, TEAM>;
     ROCM_CALL(grantDynamicLds(reinterpret_cast<const void*>(kernel), static_cast<int>(ldsBytes)));
-    hipLaunchKernelGGL(kernel, dim3(numParts), dim3(kBwdTeam * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2);
+    hipLaunchKernelGGL(kernel, dim3(numParts), dim3(TEAM * GROUPS), ldsBytes, stream, gIn, partW, partB, dout, in, w, invRms, n1, n2);
     ROCM_LAUNCH_CHECK();
     return diopiSuccess;
 }
@@ -699,23 +698,27 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     //   fp32 [32768, 1024] (NVT 1): 67.5 against 63.4 us; bf16 [8192, 4096] (NVT 2): 37.8 against 36.7 us
     //   bf16 [4096, 8192] (NVT 4): one group of two teams 46.3 us against 108.9 us for four teams, whose 16 waves leave a lane
     //   128 registers where the kernel wants 217
-    // so fp32 NVT 4 takes two groups of two teams per unit, fewer packets one group of four; 16-bit NVT 4 (217 registers) and
-    // fp32 rows of up to 8192 columns (NVT 8, 64 KiB per team array, 236 registers) one group of two.  With grad_bias a team
-    // has two arrays: one group of two teams (one of one team at NVT 8).
+    // so fewer packets than four take one group of four teams; 16-bit NVT 4 (217 registers) and fp32 rows of up to 8192 columns
+    // (NVT 8, 64 KiB per team array, 236 registers) one group of two.  With grad_bias a team has two arrays: one group of two
+    // teams (one of one team at NVT 8).  fp32 NVT 4 is the one shape that takes teams of 512 threads, see below.
     constexpr int kMaxNvt = sizeof(T) == 4 ? 8 : 4;
     if (nvec > static_cast<int64_t>(kMaxNvt) * kBwdTeam) return diopiSuccess;
     if (deviceInfo().maxSharedOptin < 128 * 1024 + 1024) return diopiSuccess;
     if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
     const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
     const int nvc = nvt <= 1 ? 1 : (nvt <= 2 ? 2 : (nvt <= 4 ? 4 : 8));
-    // (fp32 NVT 4 with fewer than 16 rows per compute unit: one group of four again, 23.2 against 25.9 us at [2048, 4096], where
-    // the second partial row per unit costs more than the faster stream brings)
-    const bool twoPerUnit = !gBias && nvc == 4 && sizeof(T) == 4 && d.n1 >= 16 * static_cast<int64_t>(deviceInfo().numCU);
-    const int groups = gBias ? (nvc == 8 ? 1 : 2) : ((nvc <= 2 || (nvc == 4 && sizeof(T) == 4 && !twoPerUnit)) ? 4 : 2);
-    const int perUnit = twoPerUnit ? 2 : 1;
-    // as many work-groups as fit the compute units (fewer when there are not enough rows to give every team one)
-    const int64_t maxBlocks = static_cast<int64_t>(deviceInfo().numCU) * perUnit;
-    const int numParts = static_cast<int>(std::min<int64_t>(maxBlocks, ceilDiv(d.n1, groups)));
+    // fp32 rows of 4 packets per thread of a 256-thread team go to teams of 512 threads with 2 packets each (fewer requests
+    // of a lane in flight and more lanes stream faster): [8192, 4096] 69.9 us against 71.7 for two work-groups of two
+    // 256-thread teams per unit, [16384, 4096] 135.2 against 137.0, with grad_bias 70.9 against 73.1; 16-bit rows of that
+    // many packets gain nothing from it (43.3 against 43.5 us at bf16 [4096, 8192]) and keep their teams.  With fewer than
+    // 16 rows per compute unit and no grad_bias: one group of four 256-thread teams (21.2 us at [2048, 4096]).
+    const bool wideTeam = nvc == 4 && sizeof(T) == 4 && (gBias != nullptr || d.n1 >= 16 * static_cast<int64_t>(deviceInfo().numCU));
+    // teams of a work-group: each owns rows of its own
+    const int groups = wideTeam ? (gBias ? 1 : 2) : (gBias ? (nvc == 8 ? 1 : 2) : ((nvc <= 2 || (nvc == 4 && sizeof(T) == 4)) ? 4 : 2));
+    // as many work-groups as there are compute units (fewer when there are not enough rows to give every team one)
+    const int64_t maxBlocks = deviceInfo().numCU;
+    const int teamsPerGroup = groups;
+    const int numParts = static_cast<int>(std::min<int64_t>(maxBlocks, ceilDiv(d.n1, teamsPerGroup)));
     const int n2 = static_cast<int>(d.n2);
     const int64_t partBytes = static_cast<int64_t>(numParts) * n2 * sizeof(float);
     void* scratch = nullptr;
@@ -727,35 +730,39 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     const T* pin = static_cast<const T*>(in.data);
     const T* pw = static_cast<const T*>(w.data);
     const float* pinv = static_cast<const float*>(invRms.data);
-#define ROCM_BWD_CASE(NVC, GB, GROUPS, WGS) \
-    ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, GB, GROUPS, WGS>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)))
+#define ROCM_BWD_CASE(NVC, GB, GROUPS, TEAM) \
+    ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, GB, GROUPS, TEAM>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)))
     if (gBias != nullptr) {
         if (nvc == 1) {
-            ROCM_BWD_CASE(1, true, 2, 1);
+            ROCM_BWD_CASE(1, true, 2, 256);
         } else if (nvc == 2) {
-            ROCM_BWD_CASE(2, true, 2, 1);
+            ROCM_BWD_CASE(2, true, 2, 256);
         } else if (nvc == 4) {
-            ROCM_BWD_CASE(4, true, 2, 1);
+            if constexpr (sizeof(T) == 4) {
+                ROCM_BWD_CASE(2, true, 1, 512);
+            } else {
+                ROCM_BWD_CASE(4, true, 2, 256);
+            }
         } else if constexpr (kMaxNvt >= 8) {
-            ROCM_BWD_CASE(8, true, 1, 1);
+            ROCM_BWD_CASE(8, true, 1, 256);
         }
     } else {
         if (nvc == 1) {
-            ROCM_BWD_CASE(1, false, 4, 1);
+            ROCM_BWD_CASE(1, false, 4, 256);
         } else if (nvc == 2) {
-            ROCM_BWD_CASE(2, false, 4, 1);
+            ROCM_BWD_CASE(2, false, 4, 256);
         } else if (nvc == 4) {
             if constexpr (sizeof(T) == 4) {
-                if (twoPerUnit) {
-                    ROCM_BWD_CASE(4, false, 2, 2);
+                if (wideTeam) {
+                    ROCM_BWD_CASE(2, false, 2, 512);
                 } else {
-                    ROCM_BWD_CASE(4, false, 4, 1);
+                    ROCM_BWD_CASE(4, false, 4, 256);
                 }
             } else {
-                ROCM_BWD_CASE(4, false, 2, 1);
+                ROCM_BWD_CASE(4, false, 2, 256);
             }
         } else if constexpr (kMaxNvt >= 8) {
-            ROCM_BWD_CASE(8, false, 2, 1);
+            ROCM_BWD_CASE(8, false, 2, 256);
         }
     }
 #undef ROCM_BWD_CASE
