@@ -259,7 +259,7 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 
 // ---------------------------------------------------------------------------
 // Backward, fused single pass (T = dtype of x, dout, weight, grad_input, grad_weight).
-// A work-group is GROUPS row teams of TEAM threads (256, or 512 for fp32 rows of 1024 packets), one work-group per compute
+// A work-group is GROUPS row teams of TEAM threads (256, 512 or 1024: the launcher says when), one work-group per compute
 // unit.  In step i, team g of work-group b takes row
 // (i * gridDim.x + b) * GROUPS + g: at any moment the whole grid works on one contiguous window of
 // gridDim.x * GROUPS rows of each tensor, which spreads the traffic evenly over the memory channels (a private run of
@@ -279,9 +279,9 @@ __global__ __launch_bounds__(kFwdThreads) void rmsNormFwdGeneric(TOut* __restric
 // the team arrays are summed in a fixed order into one fp32 partial row per work-group (one rounding of a sum that the
 // fold then continues in fp64: the error stays below one rounding of the fp32 result).  The fewer packets of a row a thread
 // holds, the faster the rows stream: at fp32 [8192, 4096] one work-group of four 256-thread teams (4 packets a thread)
-// moves the rows at 5.79 TB/s, two work-groups of two such teams per unit at 6.07, and one work-group of two 512-thread
-// teams (2 packets a thread, one partial row per unit) is another 2.5 % faster over the whole operator.  The row sum s[r]
-// crosses the team's waves through LDS: one barrier per step.
+// moves the rows at 5.79 TB/s, two work-groups of two such teams per unit at 6.07, one work-group of two 512-thread teams
+// (2 packets a thread, one partial row per unit) is another 2.5 % faster over the whole operator and one team of 1024
+// threads (1 packet a thread) 2 % more.  The row sum s[r] crosses the team's waves through LDS: one barrier per step.
 // ---------------------------------------------------------------------------
 constexpr int kBwdTeam = 256;  // threads of a team unless a shape asks for more
 constexpr int kBwdFlush = 8;
@@ -700,21 +700,26 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     //   128 registers where the kernel wants 217
     // so fewer packets than four take one group of four teams; 16-bit NVT 4 (217 registers) and fp32 rows of up to 8192 columns
     // (NVT 8, 64 KiB per team array, 236 registers) one group of two.  With grad_bias a team has two arrays: one group of two
-    // teams (one of one team at NVT 8).  fp32 NVT 4 is the one shape that takes teams of 512 threads, see below.
+    // teams (one of one team at NVT 8).  Wider teams where they pay: see below.
     constexpr int kMaxNvt = sizeof(T) == 4 ? 8 : 4;
     if (nvec > static_cast<int64_t>(kMaxNvt) * kBwdTeam) return diopiSuccess;
     if (deviceInfo().maxSharedOptin < 128 * 1024 + 1024) return diopiSuccess;
     if (!aligned16(in.data) || !aligned16(dout.data) || !aligned16(gIn.data) || !aligned16(w.data)) return diopiSuccess;
     const int nvt = static_cast<int>(ceilDiv(nvec, kBwdTeam));
     const int nvc = nvt <= 1 ? 1 : (nvt <= 2 ? 2 : (nvt <= 4 ? 4 : 8));
-    // fp32 rows of 4 packets per thread of a 256-thread team go to teams of 512 threads with 2 packets each (fewer requests
-    // of a lane in flight and more lanes stream faster): [8192, 4096] 69.9 us against 71.7 for two work-groups of two
-    // 256-thread teams per unit, [16384, 4096] 135.2 against 137.0, with grad_bias 70.9 against 73.1; 16-bit rows of that
-    // many packets gain nothing from it (43.3 against 43.5 us at bf16 [4096, 8192]) and keep their teams.  With fewer than
-    // 16 rows per compute unit and no grad_bias: one group of four 256-thread teams (21.2 us at [2048, 4096]).
-    const bool wideTeam = nvc == 4 && sizeof(T) == 4 && (gBias != nullptr || d.n1 >= 16 * static_cast<int64_t>(deviceInfo().numCU));
+    // The fewer packets of a row a thread holds, the faster the rows stream.  With at least 16 rows per compute unit and no
+    // grad_bias, rows of more than 256 packets therefore go to the widest team they fill, 1024 threads in all (us, teams of
+    // 256 threads as above -> wide teams):
+    //   fp32 [8192, 4096] 71.7 -> 68.6 (two teams of 512: 69.9), [16384, 4096] 137.0 -> 130.2, [4096, 8192] 78.4 -> 76.0
+    //   bf16 [8192, 4096] 39.8 -> 39.3, [16384, 4096] 71.3 -> 69.5, [4096, 8192] 43.5 -> 42.9
+    // With fewer rows the wide teams lose ([2048, 4096]: fp32 21.1 -> 23.3, bf16 16.0 -> 16.9: too few teams to spread the rows
+    // over), and with grad_bias they change nothing (fp32 [8192, 4096] 71.0 -> 71.1) or lose (bf16 43.2 -> 43.6), except that
+    // fp32 rows of 1024 packets take one team of 512 threads there (73.1 -> 70.9).
+    const bool manyRows = d.n1 >= 16 * static_cast<int64_t>(deviceInfo().numCU);
+    const bool wide = gBias == nullptr && manyRows && nvec > 256;
+    const bool wideBias = gBias != nullptr && nvc == 4 && sizeof(T) == 4;
     // teams of a work-group: each owns rows of its own
-    const int groups = wideTeam ? (gBias ? 1 : 2) : (gBias ? (nvc == 8 ? 1 : 2) : ((nvc <= 2 || (nvc == 4 && sizeof(T) == 4)) ? 4 : 2));
+    const int groups = wide ? (nvec <= 512 ? 2 : 1) : (wideBias ? 1 : (gBias ? (nvc == 8 ? 1 : 2) : ((nvc <= 2 || (nvc == 4 && sizeof(T) == 4)) ? 4 : 2)));
     // as many work-groups as there are compute units (fewer when there are not enough rows to give every team one)
     const int64_t maxBlocks = deviceInfo().numCU;
     const int teamsPerGroup = groups;
@@ -732,7 +737,15 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
     const float* pinv = static_cast<const float*>(invRms.data);
 #define ROCM_BWD_CASE(NVC, GB, GROUPS, TEAM) \
     ROCM_CALL((launchBwdInstance<T, ColAcc, NVC, GB, GROUPS, TEAM>(stream, numParts, pgi, partW, partB, pdo, pin, pw, pinv, d.n1, n2)))
-    if (gBias != nullptr) {
+    if (wide) {
+        if (nvec <= 512) {
+            ROCM_BWD_CASE(1, false, 2, 512);
+        } else if (nvec <= 1024) {
+            ROCM_BWD_CASE(1, false, 1, 1024);
+        } else if constexpr (kMaxNvt >= 8) {
+            ROCM_BWD_CASE(2, false, 1, 1024);
+        }
+    } else if (gBias != nullptr) {
         if (nvc == 1) {
             ROCM_BWD_CASE(1, true, 2, 256);
         } else if (nvc == 2) {
@@ -753,11 +766,7 @@ diopiError_t launchBwdFused(diopiContextHandle_t ctx, hipStream_t stream, const 
             ROCM_BWD_CASE(2, false, 4, 256);
         } else if (nvc == 4) {
             if constexpr (sizeof(T) == 4) {
-                if (wideTeam) {
-                    ROCM_BWD_CASE(2, false, 2, 512);
-                } else {
-                    ROCM_BWD_CASE(4, false, 4, 256);
-                }
+                ROCM_BWD_CASE(4, false, 4, 256);
             } else {
                 ROCM_BWD_CASE(4, false, 2, 256);
             }
