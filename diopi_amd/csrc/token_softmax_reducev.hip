@@ -226,8 +226,10 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         }
         waveLdsFence();
     };
-    // two sets of 8 rows per lane: while the products of one step consume a set, the rows of the next step are in flight
-    u32x4 rowsA[8], rowsB[8];
+    // One set of 8 rows per lane, requested a step ahead; what hides the wait of a wave is the other waves of its SIMD, not a
+    // second set in its own registers (two sets, requested two steps ahead, measured 0.8 % slower at 64 sequences of 512..2048
+    // tokens and 0.4 % at 128 of 1024..8192 with grouped heads: fewer requests of a lane in flight stream faster here).
+    u32x4 rowsV8[8];
     auto issueV = [&](int step, u32x4 (&rows)[8]) {
         const int first = 32 * step + 8 * q;
         const u32x4 s0 = *reinterpret_cast<const u32x4*>(slotW + first);
@@ -238,7 +240,6 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
             rows[4 + r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vHead + static_cast<int64_t>(static_cast<int32_t>(s1[r])) * rowStride));
         }
     };
-    static_assert((kSub / kStep) % 2 == 0, "a set of row registers keeps its parity from one sub-tile to the next");
     auto stepsOf = [&](int sub) {
         const int n = (nTokR - subOff(sub) < kSub) ? nTokR - subOff(sub) : kSub;
         return (n + kStep - 1) / kStep;
@@ -250,8 +251,7 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
         loadSlots(0);
         loadLogits(0);
         storeSlots();
-        issueV(0, rowsA);
-        if (stepsOf(0) > 1) issueV(1, rowsB);
+        issueV(0, rowsV8);
     }
 
     f32x4 acc[8];
@@ -323,23 +323,16 @@ __global__ __launch_bounds__(kRvThreads, 2) void softmaxReduceVWave(T* __restric
                 acc[2 * j] = Ops::mma(pa.f, lo.f, acc[2 * j]);
                 acc[2 * j + 1] = Ops::mma(pa.f, hi.f, acc[2 * j + 1]);
             }
-            // this set of row registers is free again: request the rows two steps ahead (of this sub-tile or of the
-            // next one, whose slots take over the wave's LDS line once the last rows of this sub-tile are requested)
-            if (s + 2 < nSteps) {
-                issueV(s + 2, rowsV);
-            } else if (s + 2 - nSteps < nStepsNext) {
-                if (s + 2 == nSteps) storeSlots();
-                issueV(s + 2 - nSteps, rowsV);
+            // the row registers are free again: request the rows of the next step (of this sub-tile or of the next one,
+            // whose slots take over the wave's LDS line once the last rows of this sub-tile are requested)
+            if (s + 1 < nSteps) {
+                issueV(s + 1, rowsV);
+            } else if (s + 1 - nSteps < nStepsNext) {
+                if (s + 1 == nSteps) storeSlots();
+                issueV(s + 1 - nSteps, rowsV);
             }
         };
-        // the first two steps run outside the loop: they wait for rows requested before the softmax and the prefetches
-        // above, the later steps for rows requested two steps earlier
-        pvStep(0, rowsA);
-        if (nSteps > 1) pvStep(1, rowsB);
-        for (int s = 2; s < nSteps; s += 2) {
-            pvStep(s, rowsA);
-            if (s + 1 < nSteps) pvStep(s + 1, rowsB);
-        }
+        for (int s = 0; s < nSteps; ++s) pvStep(s, rowsV8);
     }
 
     // ---- the waves of the work-group hand their (maximum, denominator, sums) over in LDS; all threads combine them ----
