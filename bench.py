@@ -121,17 +121,20 @@ def token_attention_floor(args, torch, rt, W, impl, ctx, check):
         for nt in (0, 4):
             for tt in (128, 256):
                 us = timed(lambda: gather(1 + nt, H, split, tt))
+                us_few = timed(lambda: gather(1 + nt + 8, H, split, tt))
                 say(what="gather only", row_bytes_per_work_group=row_bytes // split, non_temporal=bool(nt), tile_tokens=tt, us=round(us, 1),
-                    GBs=round(read_bytes / us / 1e3, 1))
+                    GBs=round(read_bytes / us / 1e3, 1), us_two_loads_in_flight=round(us_few, 1))
                 if tt == tile and (best is None or us < best[0]):
                     best = (us, split, nt)
     _, split, nt = best
     for pieces in (2 * H, H, H // 2, H // 4, H // 16, 1):
         piece_bytes = tile * H * e // pieces
         us_both = timed(lambda: gather(3 + nt, pieces, split))
+        us_few = timed(lambda: gather(3 + nt + 8, pieces, split))
         us_wr = timed(lambda: gather(2, pieces, split))
         say(what="gather + logits-sized write", row_bytes_per_work_group=row_bytes // split, non_temporal=bool(nt), piece_bytes=piece_bytes,
-            interface_layout=(pieces == H), us=round(us_both, 1), GBs=round((read_bytes + write_bytes) / us_both / 1e3, 1), write_only_us=round(us_wr, 1))
+            interface_layout=(pieces == H), us=round(us_both, 1), GBs=round((read_bytes + write_bytes) / us_both / 1e3, 1),
+            us_two_loads_in_flight=round(us_few, 1), write_only_us=round(us_wr, 1))
     wgs = 8 * int(rt.libs().rt.diopirtDeviceComputeUnits(0))
     us = timed(lambda: lib.diopiProbeCopy(stream, dst.data_ptr(), src.data_ptr(), read_bytes, wgs))
     say(what="plain copy of the read volume", us=round(us, 1), GBs=round(2 * read_bytes / us / 1e3, 1))

@@ -10,7 +10,9 @@
 // `pieces` equal runs of consecutive bytes that lie `pieceStride` bytes apart (pieces = H is the operator's own layout: one
 // run per head; fewer pieces of more bytes each are what another output layout would give).  `rowSplit` work-groups share a
 // tile: each reads its 1/rowSplit of every row (the operator gives a work-group some of the kv heads) and writes every
-// rowSplit-th piece.  Modes: 1 reads only, 2 writes only, 3 both; + 4 makes the reads non-temporal.
+// rowSplit-th piece.  Modes: 1 reads only, 2 writes only, 3 both; + 4 makes the reads non-temporal; + 8 gives a thread two
+// loads in flight instead of sixteen (more work-groups then cover for each other's waits: which of the two is faster depends
+// on the pattern, so the caller tries both).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -20,7 +22,6 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int kBatch = 8;  // loads a thread issues before it looks at the first of them; two such batches are in flight
 
 struct GatherArgs {
     const char* cache;       // [slots][rowBytes]
@@ -38,7 +39,8 @@ struct GatherArgs {
     int mode;
 };
 
-template <bool NT>
+// kBatch: loads a thread issues before it looks at the first of them; two such batches are in flight
+template <bool NT, int kBatch>
 __global__ __launch_bounds__(kThreads) void probeTokenGather(GatherArgs a) {
     // x runs over the parts of a row, y over the sequences, z over the tiles, with the sequence rotated by the tile index:
     // work-groups that start together read neighbouring parts of the same rows and tiles of many sequences, and the
@@ -222,7 +224,7 @@ extern "C" int diopiProbeTokenGather(void* stream, int mode, const void* cache, 
     if (rowSplit <= 0 || rowBytes % rowSplit != 0) return 1;
     const int partBytes = rowBytes / rowSplit;
     const bool rowOk = partBytes >= 16 && partBytes <= 16 * kThreads && (partBytes & (partBytes - 1)) == 0;
-    if (!rowOk || (mode & 3) == 0 || mode > 7 || batch <= 0 || batch > 65535 || maxLength <= 0 || tileTokens <= 0 || pieces <= 0 || bytesPerToken % pieces != 0 ||
+    if (!rowOk || (mode & 3) == 0 || mode > 15 || batch <= 0 || batch > 65535 || maxLength <= 0 || tileTokens <= 0 || pieces <= 0 || bytesPerToken % pieces != 0 ||
         (tileTokens * (bytesPerToken / pieces)) % 16 != 0 || pieceStride % 16 != 0)
         return 1;
     GatherArgs a;
@@ -242,10 +244,17 @@ extern "C" int diopiProbeTokenGather(void* stream, int mode, const void* cache, 
     const dim3 grid(static_cast<unsigned>(rowSplit), static_cast<unsigned>(batch), static_cast<unsigned>((maxLength + tileTokens - 1) / tileTokens));
     if (tileTokens > 8192) return 1;  // the slots of a tile in LDS
     const size_t lds = static_cast<size_t>(tileTokens) * sizeof(int32_t);
-    if (mode & 4) {
-        hipLaunchKernelGGL(probeTokenGather<true>, grid, dim3(kThreads), lds, static_cast<hipStream_t>(stream), a);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (mode & 8) {
+        if (mode & 4) {
+            hipLaunchKernelGGL((probeTokenGather<true, 1>), grid, dim3(kThreads), lds, s, a);
+        } else {
+            hipLaunchKernelGGL((probeTokenGather<false, 1>), grid, dim3(kThreads), lds, s, a);
+        }
+    } else if (mode & 4) {
+        hipLaunchKernelGGL((probeTokenGather<true, 8>), grid, dim3(kThreads), lds, s, a);
     } else {
-        hipLaunchKernelGGL(probeTokenGather<false>, grid, dim3(kThreads), lds, static_cast<hipStream_t>(stream), a);
+        hipLaunchKernelGGL((probeTokenGather<false, 8>), grid, dim3(kThreads), lds, s, a);
     }
     return hipGetLastError() == hipSuccess ? 0 : 1;
 }

@@ -38,7 +38,7 @@ def test_probe_library_loads_and_refuses_bad_arguments():
         return lib.diopiProbeTokenGather(None, a["mode"], None, a["row"], None, a["mil"], None, None, a["batch"], a["maxlen"], None, a["stride"], a["pieces"],
                                          a["bpt"], a["tile"], a["split"])
 
-    assert gather(mode=0) == 1 and gather(mode=8) == 1 and gather(mode=4) == 1
+    assert gather(mode=0) == 1 and gather(mode=8) == 1 and gather(mode=4) == 1 and gather(mode=16) == 1
     assert gather(row=2000) == 1                # a part of a row is 16 bytes times a power of two
     assert gather(split=3) == 1
     assert gather(pieces=3) == 1                # the bytes of a token divide evenly over the pieces
@@ -66,7 +66,7 @@ def test_gather_probe_writes_the_bytes_of_its_tiles_and_nothing_else():
         per_token = heads * e // pieces
         stride = (total * per_token + 15) // 16 * 16 + 64
         out = torch.zeros(pieces * stride, dtype=torch.uint8, device=dev)
-        for mode in (2, 3, 7):
+        for mode in (2, 3, 7, 15):
             out.zero_()
             assert lib.diopiProbeTokenGather(stream, mode, cache.data_ptr(), row_bytes, loc.data_ptr(), mil, start.data_ptr(), length.data_ptr(), B, max(lengths),
                                              out.data_ptr(), stride, pieces, heads * e, tile, split) == 0
